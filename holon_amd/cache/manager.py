@@ -5,8 +5,8 @@ State that grows lives in pages. Paged states of equal page geometry (values per
 declare them and however many one run declares, form a *group*: one page pool, one block table, one storage tensor
 `[members, pages, page_size * elems]` with a member for every (run, state name) of the group. Page id p means row p
 of every member. Groups with different needs (all tokens, a window of them, another width) have pools and tables of
-their own; a windowed group gives pages back as soon as the window has passed them, a finished request gives back
-everything.
+their own; a windowed group gives pages back as soon as the window has passed them (all but the pages of the first
+tokens, where the declaration says that those stay visible), a finished request gives back everything.
 
 With a prefix index (`enable_prefix`) full pages of tokens are shared between requests that start alike: `adopt` gives
 a new request the cached pages of its longest known prefix, `publish` hands the pages a request has filled to the
@@ -38,8 +38,10 @@ class PagedGroup:
     storage: torch.Tensor                         # [len(members), num_pages, page_size * elems]
     table: np.ndarray                             # [max_seqs + 1, max_pages] int32, null page where nothing is held
     table_dev: torch.Tensor
-    first: list[int]                              # per slot: first page index still held
-    count: list[int]                              # per slot: page indices [first, count) are held
+    first: list[int]                              # per slot: first page index of the window still held
+    count: list[int]                              # per slot: page indices [first, count) are held, and beside them
+    kept: int = 0                                 # the first `kept` pages of the sequence (a window that keeps its
+                                                  # first tokens): held are [0, min(kept, first)) and [first, count)
     dirty: set[int] = dataclasses.field(default_factory=set)
 
 
@@ -72,7 +74,7 @@ class CacheManager:
                 raise ValueError(f"run {site.run} declares two states of one name: {names}")
             for d in site_decls:
                 if isinstance(d, PagedState):
-                    key = (d.elems, d.window, d.dtype or dtype)
+                    key = (d.elems, d.window, d.dtype or dtype, d.keep_first if d.window > 0 else 0)
                     keyed.setdefault(key, []).append((site.run, d.name))
                 elif isinstance(d, SlotState):
                     t = torch.zeros((max_seqs + 1, *d.shape), dtype=d.dtype or dtype, device=device)
@@ -80,13 +82,14 @@ class CacheManager:
                     self.slot_states.append((site.run, d, t))
                 else:
                     raise TypeError(f"run {site.run}: unknown state declaration {d!r}")
-        for gid, ((elems, window, gdtype), members) in enumerate(keyed.items()):
+        for gid, ((elems, window, gdtype, keep_first), members) in enumerate(keyed.items()):
             pool = PagePool(num_pages)
             storage = torch.zeros((len(members), num_pages, page_size * elems), dtype=gdtype, device=device)
             table = np.full((max_seqs + 1, self.max_pages), pool.null, dtype=np.int32)
             runs = sorted({run for run, _ in members})
-            group = PagedGroup(gid, PagedState("", elems, window, gdtype), runs, members, pool, storage, table,
-                               torch.from_numpy(table.copy()).to(device), [0] * (max_seqs + 1), [0] * (max_seqs + 1))
+            group = PagedGroup(gid, PagedState("", elems, window, gdtype, keep_first), runs, members, pool, storage,
+                               table, torch.from_numpy(table.copy()).to(device), [0] * (max_seqs + 1),
+                               [0] * (max_seqs + 1), kept=-(-keep_first // page_size))
             self.groups.append(group)
             for at, (run, name) in enumerate(members):
                 sites[run].paged[name] = SitePages(gid, storage[at])
@@ -122,7 +125,7 @@ class CacheManager:
         if slot not in self._live:
             raise RuntimeError(f"slot {slot} released twice (or never admitted)")
         for g in self.groups:
-            for i in range(g.first[slot], g.count[slot]):
+            for i in self._held(g, slot):
                 g.pool.decref(int(g.table[slot, i]))
             g.table[slot, : g.count[slot]] = g.pool.null
             g.first[slot] = g.count[slot] = 0
@@ -131,6 +134,12 @@ class CacheManager:
         self.computed[slot] = self._capacity[slot] = 0
         self.chain[slot] = None
         self._free_slots.append(slot)
+
+    @staticmethod
+    def _held(g: PagedGroup, slot: int) -> list[int]:
+        """The page indices of a slot's table that hold pages: the kept first pages and the window's."""
+        first, count = g.first[slot], g.count[slot]
+        return list(range(min(g.kept, first, count))) + list(range(first, count))
 
     # -- shared prefixes ------------------------------------------------------------------------------------------
     def enable_prefix(self, namespace: bytes) -> bool:
@@ -246,11 +255,13 @@ class CacheManager:
             keep_from = max(0, computed - w + 1) // self.page_size      # the next query reads keys from computed-w+1
             keep_from = min(keep_from, g.count[slot])
             if keep_from > g.first[slot]:
-                for i in range(g.first[slot], keep_from):
+                gone = range(max(g.first[slot], g.kept), keep_from)      # the first tokens' pages stay
+                for i in gone:
                     g.pool.decref(int(g.table[slot, i]))
-                g.table[slot, g.first[slot]: keep_from] = g.pool.null
+                if len(gone):
+                    g.table[slot, gone.start: gone.stop] = g.pool.null
+                    g.dirty.add(slot)
                 g.first[slot] = keep_from
-                g.dirty.add(slot)
 
     def could_fit(self, slot: int | None, total: int, victims: list[int]) -> bool:
         """Whether releasing the requests in `victims` (slots) would let `slot` (None: a new request) keep `total`
@@ -259,11 +270,11 @@ class CacheManager:
         for gid, g in enumerate(self.groups):
             have = g.count[slot] if slot is not None else 0
             if self.prefix is None:
-                freed = sum(g.count[v] - g.first[v] for v in victims)
+                freed = sum(len(self._held(g, v)) for v in victims)
             else:                       # a page comes free when only the index, or nobody, would still hold it
                 dropped: dict[int, int] = {}
                 for v in victims:
-                    for p in g.table[v, g.first[v]: g.count[v]].tolist():
+                    for p in g.table[v, self._held(g, v)].tolist():
                         dropped[p] = dropped.get(p, 0) + 1
                 cached = self.prefix.is_cached(gid)
                 freed = sum(1 for p in cached if g.pool.refs(p) - dropped.get(p, 0) == 1)
@@ -327,8 +338,9 @@ class CacheManager:
             held: dict[int, int] = {}
             for slot in range(self.max_seqs + 1):
                 row = g.table[slot]
-                inside = row[g.first[slot]: g.count[slot]]
-                outside = np.concatenate((row[: g.first[slot]], row[g.count[slot]:]))
+                held_at = np.zeros(row.shape[0], dtype=bool)
+                held_at[self._held(g, slot)] = True
+                inside, outside = row[held_at], row[~held_at]
                 if slot not in self._live and g.count[slot]:
                     raise AssertionError(f"group {g.gid}: free slot {slot} holds pages")
                 if (outside != g.pool.null).any() or (inside == g.pool.null).any():

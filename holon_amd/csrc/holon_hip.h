@@ -268,11 +268,28 @@ int holon_dyt_stream(void* x, int x_dtype, const void* term, int term_dtype, con
 
 // -- softmax attention with a window and a sink over pages of keys [Hkv, P, D] then values [Hkv, V, P] ------------------
 // (softmax_attention.hip) q [T, H, D] -> out [T, H V]; token t reads block table row slots[token_row[t]] and stands at
-// positions[t]; sink [H] float32 or null; window 0: everything before.
+// positions[t]; sink [H] float32 or null; window 0: everything before. softcap > 0: scores become softcap tanh(s /
+// softcap); r1, r2 [H] float32 (both or neither): r1 ln(1 + r2 (i - j)) is taken off the score of key j for query i;
+// keep_first: under a window, keys 0 .. keep_first - 1 stay visible.
 int holon_softmax_attention(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
                             int table_rows, const int32_t* slots, const int32_t* token_row, const int32_t* positions,
                             int tokens, int heads, int kv_heads, int dim, int vdim, int page_size, int num_pages,
-                            const float* sink, float scale, int window, int dtype, void* stream);
+                            const float* sink, float scale, int window, int dtype, float softcap, const float* r1,
+                            const float* r2, int keep_first, void* stream);
+// qkv [T, H D + G D + G V]: the query values of a token RMS-normed as one vector with q_weight [H D], its key values
+// with k_weight [G D]; queries to q [T, H, D], keys and values into the token's page.
+int holon_whole_norm_prepare(const void* qkv, int tokens, int heads, int kv_heads, int dim, int vdim,
+                             const void* q_weight, const void* k_weight, float eps, void* q, void* pages,
+                             const int32_t* write_page, const int32_t* write_off, int page_size, int num_pages, int dtype,
+                             void* stream);
+// both [T, H (dim + rot) + kv_rank + rot]: the latent RMS-normed, the first rd of every rotated part's rot dimensions
+// turned by the position (table [table_rows, rd] float32: cosines, then sines); unrotated query parts to qn [T, H, dim],
+// rotated ones into the last rot columns of full [T, H, kv_rank + rot]; [latent, rotated key part] into the token's
+// page as a key row and as a value column.
+int holon_latent_rope_prepare(const void* both, int tokens, int heads, int dim, int rot, int kv_rank,
+                              const void* c_weight, float eps, const float* table, int rd, int table_rows,
+                              const int32_t* positions, void* qn, void* full, void* pages, const int32_t* write_page,
+                              const int32_t* write_off, int page_size, int num_pages, int dtype, void* stream);
 
 // The latent attention's two latents, side by side in `both` [T, q_rank + kv_rank]: each divided by its root mean square
 // and multiplied by its weight; the first to cq [T, q_rank], the second into the token's page as a key row and as a
@@ -280,9 +297,33 @@ int holon_softmax_attention(const void* q, void* out, const void* pages, const i
 int holon_latent_prepare(const void* both, int tokens, int q_rank, int kv_rank, const void* q_weight,
                          const void* c_weight, float eps, void* cq, void* pages, const int32_t* write_page,
                          const int32_t* write_off, int page_size, int num_pages, int dtype, void* stream);
-// y [rows, H, B] = x [rows, H, A] times every head's own w [H, B, A], for steps of up to 16 rows.
-int holon_head_linear_rows(const void* x, const void* w, void* y, int rows, int heads, int A, int B, int dtype,
-                           void* stream);
+// y [rows, H, B] = x [rows, H, A] times every head's own w [H, B, A], for steps of up to 16 rows; a head's results lie
+// y_head values apart (B, or more where y is part of wider rows).
+int holon_head_linear_rows(const void* x, const void* w, void* y, int rows, int heads, int A, int B, int y_head,
+                           int dtype, void* stream);
+
+// -- a block of two sublayers over one float32 stream (parallel_block.hip) ----------------------------------------------
+// x32 [rows, dim] += (d1 + d2) + row in place (each nullable; d1, d2 float32 or bfloat16 by dt1, dt2; row [dim] float32);
+// then, with w1 and y1: y1 = x rsqrt(mean(x^2) + eps) w1, and with w2 and y2 the same rows with w2 (weights of dtype dtw,
+// results of dt_out).
+int holon_stream_rms(float* x32, const void* d1, int dt1, const void* d2, int dt2, const float* row, const void* w1,
+                     const void* w2, int dtw, void* y1, void* y2, int64_t rows, int dim, float eps, int dt_out,
+                     void* stream);
+// y[i] = scale * x[i] as float32 (x float32 or bfloat16): a new copy.
+int holon_scale_rows(const void* x, float* y, int64_t n, int dtype, float scale, void* stream);
+
+// -- feed-forward kinds (ffn_kinds.hip) ---------------------------------------------------------------------------------
+// y = coef[0] N(z) + coef[1] N(z^2) + coef[2] N(z^3) + coef[3] over rows of `dim`, N(v) = v / sqrt(mean(v^2) + eps).
+int holon_polynorm(const void* z, const float* coef, void* y, int64_t rows, int dim, float eps, int dtype, void* stream);
+// logits [rows, experts] float32 -> weights [rows, experts]: sigmoid scores; chosen by score + correction (nullable)
+// among the `keep` best of `groups` groups of neighbours (a group's score: its two largest choices), `top` a row;
+// a chosen expert's weight is score * scale, every other 0.
+int holon_moe_route(const float* logits, const float* correction, float* weights, int64_t rows, int experts, int top,
+                    int groups, int keep, float scale, void* stream);
+// gate_up [rows, 2 C], C = experts ff + shared: y [rows, C] = silu(gate) up times the weight of the column's expert
+// (the last `shared` columns: 1), exactly 0 where the weight is 0.
+int holon_moe_gate(const void* gate_up, const float* weights, void* y, int64_t rows, int experts, int ff, int shared,
+                   int dtype, void* stream);
 
 // -- the matrix memory of xLSTM (mlstm.hip) -------------------------------------------------------------------------------
 // proj [T, width]: q, k [H D] and v [H V] and the gates' pre-activations [2 H] (input, then forget) from the given

@@ -1,4 +1,4 @@
 """Architectures. Importing this package registers them by their config.json name."""
-from . import qwen3, relanex, tolurax
+from . import nevodra, qwen3, relanex, tolurax
 
-__all__ = ["qwen3", "relanex", "tolurax"]
+__all__ = ["nevodra", "qwen3", "relanex", "tolurax"]

@@ -32,12 +32,14 @@ class ParamDecl:
 @dataclasses.dataclass(frozen=True)
 class PagedState:
     """State that grows by `elems` values per token. Sites whose declarations are equal share a page pool and a block
-    table; a window W > 0 says that tokens more than W-1 behind the newest are never read again."""
+    table; a window W > 0 says that tokens more than W-1 behind the newest are never read again, except the first
+    `keep_first` tokens of the sequence, which are read for as long as it lives."""
 
     name: str
     elems: int
     window: int = 0
     dtype: torch.dtype | None = None              # None: the engine's dtype
+    keep_first: int = 0
 
 
 @dataclasses.dataclass(frozen=True)

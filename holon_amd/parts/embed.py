@@ -11,13 +11,18 @@ from .base import Build, EmbedPart, Part
 @register_part("embed", "table")
 class Embedding(EmbedPart):
     """Rows of a table. With `norm` (any registered norm whose `forward` takes `out_dtype`) the rows go through it
-    and come out in float32: the start of a residual stream that is kept in 32-bit."""
+    and come out in float32: the start of a residual stream that is kept in 32-bit. With `scale` the rows are
+    multiplied by it, in float32, and come out in float32 as well."""
 
     graph_safe = True
 
-    def __init__(self, build: Build, *, vocab: int, hidden: int, norm: PartRef | None = None) -> None:
+    def __init__(self, build: Build, *, vocab: int, hidden: int, norm: PartRef | None = None,
+                 scale: float | None = None) -> None:
         super().__init__(build)
         self.declare("weight", (vocab, hidden))
+        self.scale = None if scale is None else float(scale)
+        if self.scale is not None and norm is not None:
+            raise ValueError("embed table: either a norm or a scale")
         self.norm = None
         if norm is not None:
             self.attach("norm", build.make(norm, dim=hidden))
@@ -29,6 +34,9 @@ class Embedding(EmbedPart):
                 want_stats: bool = False):
         """Rows of the table; `take`: where a token is still on the device, see the kernel contract. With
         `want_stats`: (rows, their statistics for a norm that follows, or None)."""
+        if self.scale is not None:
+            rows = self.kernels.scale_rows(self.kernels.embedding(ids, self.weight, take, False), self.scale)
+            return (rows, None) if want_stats else rows
         if self.norm is None:
             return self.kernels.embedding(ids, self.weight, take, want_stats)
         rows = self.norm(self.kernels.embedding(ids, self.weight, take, False), out_dtype=torch.float32)

@@ -1,10 +1,15 @@
-"""Feed-forward parts. SwiGLU: std/holon_std/ffn/units.py:12-50, activation std/holon_std/ffn/reference.py:7-12."""
+"""Feed-forward parts. SwiGLU: std/holon_std/ffn/units.py:12-50, activation std/holon_std/ffn/reference.py:7-12.
+Beside it a dense feed-forward with the PolyNorm activation and a mixture of experts (HIP forms of their elementwise
+steps: `csrc/ffn_kinds.hip`)."""
 from __future__ import annotations
+
+import ctypes
 
 import torch
 
+from ..kernels.registry import KernelOp, register_kernel
 from ..registry import register_part
-from .base import Build, Part, Stream
+from .base import FLOAT32, Build, Part, Stream
 from .linear import Linear
 from .norms import Normed
 
@@ -47,5 +52,190 @@ class SwiGLU(Part):
         if y is None:
             y = self.kernels.silu_mul(gate_up(x))
         return self.down_proj(y, residual=residual)
+
+    __call__ = forward
+
+
+# -- a dense feed-forward with the PolyNorm activation, and a mixture of experts ------------------------------------------
+_P, _I, _L, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _need(cond: bool, what: str) -> None:
+    if not cond:
+        raise ValueError(what)
+
+
+def polynorm_plain(z, coef, eps):
+    """z [T, F], coef [4] float32 = (a, b, c, e): a N(z) + b N(z^2) + c N(z^3) + e with the powers taken element by
+    element and N(v) = v / sqrt(mean(v^2) + eps) over a row. float32 inside, one rounding to z's dtype."""
+    x = z.float()
+    a, b, c, e = coef.float().unbind(0)
+
+    def unit(v):
+        return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    return (a * unit(x) + b * unit(x * x) + c * unit(x * x * x) + e).to(z.dtype)
+
+
+def _polynorm_hip(launch, z, coef, eps):
+    _need(z.is_cuda and z.is_contiguous() and z.dim() == 2 and z.dtype in _DT and coef.is_cuda and coef.is_contiguous()
+          and coef.dtype == torch.float32 and coef.shape == (4,), "polynorm: contiguous rows and four float32 numbers")
+    y = torch.empty_like(z)
+    if z.shape[0]:
+        launch(z.data_ptr(), coef.data_ptr(), y.data_ptr(), z.shape[0], z.shape[1], float(eps), _DT[z.dtype])
+    return y
+
+
+def moe_route_plain(logits, correction, top, groups, keep, scale):
+    """Router logits [T, E] float32 -> weights [T, E] float32: s = sigmoid(logits); experts are chosen by s +
+    `correction` [E] (None: by s): the `top` largest among the experts of the `keep` best of `groups` equal groups of
+    neighbouring experts, a group's score being the sum of its two largest choice scores (groups <= 1: among all).
+    A chosen expert's weight is s * scale (the score without the correction, not renormalised), every other 0."""
+    s = torch.sigmoid(logits.float())
+    choice = s if correction is None else s + correction.float()
+    t, e = s.shape
+    if groups > 1:
+        size = e // groups
+        score = choice.view(t, groups, size).topk(min(2, size), dim=-1).values.sum(-1)
+        best = score.topk(keep, dim=-1).indices
+        open_ = torch.zeros((t, groups), dtype=torch.bool, device=s.device).scatter_(1, best, True)
+        choice = choice.masked_fill(~open_.repeat_interleave(size, dim=1), float("-inf"))
+    chosen = choice.topk(top, dim=-1).indices
+    return torch.zeros_like(s).scatter_(1, chosen, s.gather(1, chosen) * scale)
+
+
+def _moe_route_hip(launch, logits, correction, top, groups, keep, scale):
+    t, e = logits.shape
+    _need(logits.is_cuda and logits.is_contiguous() and logits.dtype == torch.float32 and 1 <= top <= e <= 1024
+          and (correction is None or (correction.dtype == torch.float32 and correction.is_contiguous()
+                                      and correction.shape == (e,)))
+          and (groups <= 1 or (e % groups == 0 and 1 <= keep <= groups)),
+          f"moe_route: {e} experts, top {top}, {groups} groups of which {keep} (float32 logits, at most 1,024 experts)")
+    w = torch.empty_like(logits)
+    if t:
+        launch(logits.data_ptr(), None if correction is None else correction.data_ptr(), w.data_ptr(), t, e, int(top),
+               int(groups), int(keep), float(scale))
+    return w
+
+
+def moe_gate_plain(gate_up, weights, ff, shared):
+    """gate_up [T, 2 C] with C = E ff + shared columns of gates, then as many of ups; weights [T, E] float32.
+    -> [T, C]: silu(gate) * up (as `silu_mul` rounds it), times the weight of the column's expert (column c belongs to
+    expert c // ff; the last `shared` columns to an expert that every token uses with weight 1); exactly 0 where the
+    weight is 0. One more rounding for the weight."""
+    t, e = weights.shape
+    c = e * ff + shared
+    g, u = gate_up[:, :c].float(), gate_up[:, c:].float()
+    act = ((g * torch.sigmoid(g)).to(gate_up.dtype).float() * u).to(gate_up.dtype)
+    w = weights.repeat_interleave(ff, dim=1)
+    if shared:
+        w = torch.cat((w, torch.ones((t, shared), dtype=w.dtype, device=w.device)), dim=1)
+    return torch.where(w == 0, torch.zeros_like(act), (act.float() * w).to(gate_up.dtype))
+
+
+def _moe_gate_hip(launch, gate_up, weights, ff, shared):
+    t, e = weights.shape
+    c = e * ff + shared
+    _need(gate_up.is_cuda and gate_up.is_contiguous() and gate_up.dtype in _DT and gate_up.shape == (t, 2 * c)
+          and weights.is_contiguous() and weights.dtype == torch.float32,
+          f"moe_gate: rows {tuple(gate_up.shape)} for {e} experts of {ff} and {shared} shared columns")
+    y = torch.empty((t, c), dtype=gate_up.dtype, device=gate_up.device)
+    if t:
+        launch(gate_up.data_ptr(), weights.data_ptr(), y.data_ptr(), t, e, ff, shared, _DT[gate_up.dtype])
+    return y
+
+
+register_kernel(KernelOp("polynorm", polynorm_plain, "holon_polynorm", [_P, _P, _P, _L, _I, _F, _I], _polynorm_hip))
+register_kernel(KernelOp("moe_route", moe_route_plain, "holon_moe_route", [_P, _P, _P, _L, _I, _I, _I, _I, _F],
+                         _moe_route_hip))
+register_kernel(KernelOp("moe_gate", moe_gate_plain, "holon_moe_gate", [_P, _P, _P, _L, _I, _I, _I, _I], _moe_gate_hip))
+
+
+@register_part("ffn", "polynorm")
+class PolyNormFFN(Part):
+    """down(act(up(x))) with act = a N(z) + b N(z^2) + c N(z^3) + e (`act` holds a, b, c, e; N divides a token's
+    vector by its root mean square, `eps` inside the root)."""
+
+    graph_safe = True
+
+    def __init__(self, build: Build, *, inter: int, eps: float, hidden: int, layer: int) -> None:
+        super().__init__(build)
+        self.inter, self.hidden, self.eps = inter, hidden, float(eps)
+        self.attach("up_proj", Linear(build, inp=hidden, out=inter))
+        self.attach("down_proj", Linear(build, inp=inter, out=hidden))
+        self.declare("act", (4,), kind=FLOAT32, init="unit")
+
+    def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
+        return self.down_proj(self.kernels.polynorm(self.up_proj(x), self.act, self.eps))
+
+    __call__ = forward
+
+
+@register_part("ffn", "moe")
+class MoE(Part):
+    """A mixture of SiLU-gated experts with a sigmoid router, and an optional shared expert that every token uses.
+
+    Router: float32 logits, scores s = sigmoid(logits); experts are chosen by s + `correction` (`bias`), optionally
+    only within the `keep` best of `groups` groups of neighbouring experts, `top` per token; a chosen expert's output
+    is weighted by s * `scale`. All experts' gate and up projections are one product and all down projections
+    another: the activations of experts a token did not choose are set to 0 in between (`moe_gate`), so the second
+    product adds up exactly the chosen experts' weighted outputs, and the shared expert's columns ride in the same two
+    products. Every step launches the same kernels whatever was chosen."""
+
+    graph_safe = True
+
+    def __init__(self, build: Build, *, experts: int, top: int, inter: int, hidden: int, layer: int,
+                 scale: float = 1.0, groups: int = 1, keep: int = 1, bias: bool = True, shared: int = 0) -> None:
+        super().__init__(build)
+        if not 1 <= top <= experts:
+            raise ValueError(f"moe: top {top} of {experts} experts")
+        if groups > 1 and (experts % groups or not 1 <= keep <= groups or top > keep * (experts // groups)):
+            raise ValueError(f"moe: {experts} experts in {groups} groups, {keep} kept, top {top}")
+        self.experts, self.top, self.inter, self.hidden, self.shared = experts, top, inter, hidden, int(shared)
+        self.scale, self.groups, self.keep = float(scale), int(groups), int(keep)
+        self.declare("router", (experts, hidden), kind=FLOAT32)
+        self.has_bias = bool(bias)
+        if self.has_bias:
+            self.declare("correction", (experts,), kind=FLOAT32, init="zero")
+        self.declare("gate", (experts, inter, hidden))
+        self.declare("up", (experts, inter, hidden))
+        self.declare("down", (experts, hidden, inter))
+        if self.shared:
+            self.declare("shared_gate", (self.shared, hidden))
+            self.declare("shared_up", (self.shared, hidden))
+            self.declare("shared_down", (hidden, self.shared))
+        self.gate_up: Linear | None = None
+        self.all_down: Linear | None = None
+
+    def finalize(self) -> None:
+        if self.gate is None:
+            return
+        e, f, w = self.experts, self.inter, self.hidden
+        cols = e * f + self.shared
+        gate_up, down = Linear(self.build, inp=w, out=2 * cols), Linear(self.build, inp=cols, out=w)
+        gates, ups = [self.gate.reshape(e * f, w)], [self.up.reshape(e * f, w)]
+        downs = [self.down.permute(1, 0, 2).reshape(w, e * f)]
+        if self.shared:
+            gates.append(self.shared_gate)
+            ups.append(self.shared_up)
+            downs.append(self.shared_down)
+        gate_up.weight = torch.cat(gates + ups, dim=0).contiguous()
+        down.weight = torch.cat(downs, dim=1).contiguous()
+        for name in ("gate", "up", "down", "shared_gate", "shared_up", "shared_down"):
+            if name in self._decls:
+                del self._decls[name]
+                setattr(self, name, None)
+        gate_up.finalize()
+        down.finalize()
+        self.gate_up = self.attach("gate_up", gate_up)
+        self.all_down = self.attach("all_down", down)
+
+    def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
+        k = self.kernels
+        logits = k.linear(x if x.dtype == torch.float32 else k.widen_rows(x), self.router)
+        weights = k.moe_route(logits, self.correction if self.has_bias else None, self.top, self.groups, self.keep,
+                              self.scale)
+        act = k.moe_gate(self.gate_up(x), weights, self.inter, self.shared)
+        return self.all_down(act)
 
     __call__ = forward

@@ -1,0 +1,197 @@
+"""A block whose two sublayers read the same residual stream, kept in float32:
+
+    x += mixer(f1(norm1(x))) + ffn(f2(norm2(x)))
+
+Both norms are RMS norms of the same rows, so they share the row's mean square and one kernel produces both results
+(`stream_rms`, HIP form in `csrc/parallel_block.hip`); the same kernel first adds what the layer before left to add
+(its two results, summed before they join the stream) and, for a block that opens a repeated range of layers, the
+vector of the pass that begins (`pass_steps`: a tensor `[passes, hidden]` whose row `site.turn` is added in front of
+every pass, the first too). f1 and f2 (`conv_taps` > 0) replace a sublayer's input a by a + conv(a), a short causal
+filter over time on every channel whose last taps - 1 inputs are part of the request's state. A layer may lack the
+feed-forward; its second norm and filter are then not built.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from ..kernels.registry import KernelOp, register_kernel
+from ..registry import register_part
+from ..spec import PartRef
+from .base import FLOAT32, Build, NormPart, Part, Stream
+from .convs import CausalConv
+from .stream32 import Pending, _terms
+
+_P, _I, _L, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _need(cond: bool, what: str) -> None:
+    if not cond:
+        raise ValueError(what)
+
+
+def stream_rms_plain(x32, terms, row, w1, w2, eps, out_dtype):
+    """x32 [T, W] float32, updated in place: x += (t1 + t2) for the `terms` [(tensor [T, W], 1.0)] (at most two, summed
+    first), then x += `row` [W] float32 (None: nothing). Then r = rsqrt(mean(x^2) + eps) per row and the answers
+    (x r w1, x r w2) in `out_dtype`, the second None when `w2` is; with `w1` None nothing is normed and (None, None)
+    comes back. float32 arithmetic, one rounding of each answer."""
+    if terms:
+        add = terms[0][0].float()
+        for t, _ in terms[1:]:
+            add = add + t.float()
+        x32.add_(add)
+    if row is not None:
+        x32.add_(row.float())
+    if w1 is None:
+        return None, None
+    unit = x32 * torch.rsqrt(x32.pow(2).mean(-1, keepdim=True) + eps)
+    return (unit * w1.float()).to(out_dtype), ((unit * w2.float()).to(out_dtype) if w2 is not None else None)
+
+
+def _stream_rms_hip(launch, x32, terms, row, w1, w2, eps, out_dtype):
+    _need(x32.is_cuda and x32.is_contiguous() and x32.dtype == torch.float32 and x32.dim() == 2,
+          "stream_rms: the stream is contiguous float32 rows on the GPU")
+    _need(len(terms) <= 2 and all(float(s) == 1.0 for _, s in terms), "stream_rms: at most two terms, unscaled")
+    rows, dim = x32.shape
+    ptrs, dts = [None, None], [0, 0]
+    for i, (term, _) in enumerate(terms):
+        _need(term.is_cuda and term.is_contiguous() and term.shape == x32.shape and term.dtype in _DT,
+              f"stream_rms: term {i} must be contiguous rows of the stream's shape")
+        ptrs[i], dts[i] = term.data_ptr(), _DT[term.dtype]
+    _need(row is None or (row.is_cuda and row.is_contiguous() and row.dtype == torch.float32 and row.shape == (dim,)),
+          "stream_rms: the added row is float32 of the stream's width")
+    y1 = y2 = None
+    for w in (w1, w2):
+        _need(w is None or (w.is_cuda and w.is_contiguous() and w.shape == (dim,) and w.dtype in _DT),
+              "stream_rms: a weight of the rows' width")
+    _need(w1 is not None or w2 is None, "stream_rms: a second weight without the first")
+    if w1 is not None:
+        _need(out_dtype in _DT, "stream_rms: float32 or bfloat16 out")
+        y1 = torch.empty((rows, dim), dtype=out_dtype, device=x32.device)
+        y2 = torch.empty((rows, dim), dtype=out_dtype, device=x32.device) if w2 is not None else None
+    if rows:
+        launch(x32.data_ptr(), ptrs[0], dts[0], ptrs[1], dts[1], _ptr(row), _ptr(w1), _ptr(w2),
+               _DT[w1.dtype] if w1 is not None else 0, _ptr(y1), _ptr(y2), rows, dim, float(eps),
+               _DT[out_dtype] if w1 is not None else 0)
+    return y1, y2
+
+
+def scale_rows_plain(x, scale):
+    """x [T, W] -> a new float32 tensor of scale * x."""
+    return x.float() * scale
+
+
+def _scale_rows_hip(launch, x, scale):
+    _need(x.is_cuda and x.is_contiguous() and x.dtype in _DT, "scale_rows: contiguous float32 or bfloat16 rows on the GPU")
+    y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    launch(x.data_ptr(), y.data_ptr(), x.numel(), _DT[x.dtype], float(scale))
+    return y
+
+
+register_kernel(KernelOp("stream_rms", stream_rms_plain, "holon_stream_rms",
+                         [_P, _P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _L, _I, _F, _I], _stream_rms_hip))
+register_kernel(KernelOp("scale_rows", scale_rows_plain, "holon_scale_rows", [_P, _P, _L, _I, _F], _scale_rows_hip))
+
+
+@register_part("norm", "rms32")
+class RMSNorm32(NormPart):
+    """y = x * rsqrt(mean(x^2) + eps) * weight over rows of a float32 stream (rows in the engine's dtype are widened
+    first); float32 inside, the result in the engine's dtype."""
+
+    graph_safe = True
+
+    def __init__(self, build: Build, *, eps: float, dim: int) -> None:
+        super().__init__(build)
+        self.eps, self.dim = float(eps), dim
+        self.declare("weight", (dim,), init="norm")
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if x.dtype != torch.float32:
+            x = self.kernels.widen_rows(x)
+        return self.kernels.stream_rms(x, [], None, self.weight, None, self.eps, self.build.dtype)[0]
+
+    __call__ = forward
+
+    def add(self, x, residual: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        """(norm(residual + x), residual + x): `residual` is float32 and takes the sum in place; `x` is a tensor or
+        `Pending` terms."""
+        return self.kernels.stream_rms(residual, _terms(x), None, self.weight, None, self.eps, self.build.dtype)[0], \
+            residual
+
+    def fusion(self) -> dict | None:
+        return {"norm": "rmsnorm", "eps": self.eps, "weight": self.weight}
+
+
+@register_part("block", "parallel32")
+class Parallel32(Part):
+    """x += mixer(f1(norm1(x))) + ffn(f2(norm2(x))) over a float32 stream; see the module's text. The norms are of
+    the kind the layer names; where both are RMS norms of one eps (`fusion()`), one kernel serves both."""
+
+    graph_safe = True
+
+    def __init__(self, build: Build, *, layer: int, hidden: int, mixer: PartRef, ffn: PartRef | None, norm: PartRef,
+                 conv_taps: int = 0, pass_steps: int = 0) -> None:
+        super().__init__(build)
+        self.hidden = hidden
+        self.attach("norm1", build.make(norm, dim=hidden))
+        self.attach("mixer", build.make(mixer, layer=layer, hidden=hidden))
+        self.conv1 = self.conv2 = self.ffn = self.norm2 = None
+        if conv_taps > 0:
+            self.attach("conv1", CausalConv(build, channels=hidden, taps=conv_taps, add_input=True, name="filter1"))
+        if ffn is not None:
+            self.attach("norm2", build.make(norm, dim=hidden))
+            self.attach("ffn", build.make(ffn, layer=layer, hidden=hidden))
+            if conv_taps > 0:
+                self.attach("conv2", CausalConv(build, channels=hidden, taps=conv_taps, add_input=True, name="filter2"))
+        self.passes = int(pass_steps)
+        if self.passes > 0:
+            self.declare("step", (self.passes, hidden), kind=FLOAT32, init="zero")
+        self._one_kernel: float | None = None      # the norms' eps when one kernel serves both
+
+    def finalize(self) -> None:
+        specs = [n.fusion() for n in (self.norm1, self.norm2) if n is not None]
+        if all(sp is not None and sp.get("norm") == "rmsnorm" and sp["weight"] is not None for sp in specs) \
+                and len({sp["eps"] for sp in specs}) == 1:
+            self._one_kernel = float(specs[0]["eps"])
+
+    def state(self):
+        return [s for conv in (self.conv1, self.conv2) if conv is not None for s in conv.state()] + \
+            list(self.mixer.state())
+
+    def forward(self, stream: Stream, step, site) -> Stream:
+        k = self.kernels
+        h = stream.h
+        if h.dtype != torch.float32 or h is stream.origin:       # the stream becomes float32 rows of its own
+            h = stream.h = k.widen_rows(h)
+        row = None
+        if self.passes > 0:
+            if site.turn >= self.passes:
+                raise ValueError(f"pass {site.turn} of a range that has vectors for {self.passes} passes")
+            row = self.step[site.turn]
+        terms = _terms(stream.delta)
+        stream.delta = stream.stats = None
+        if self._one_kernel is not None:
+            a, b = k.stream_rms(h, terms, row, self.norm1.weight, self.norm2.weight if self.norm2 is not None else None,
+                                self._one_kernel, self.build.dtype)
+        else:
+            if terms or row is not None:
+                k.stream_rms(h, terms, row, None, None, 0.0, self.build.dtype)
+            a = self.norm1(h)
+            b = self.norm2(h) if self.norm2 is not None else None
+        if self.conv1 is not None:
+            a = self.conv1(a, step, site)
+        out = [(self.mixer(a, step, site), 1.0)]
+        if self.ffn is not None:
+            if self.conv2 is not None:
+                b = self.conv2(b, step, site)
+            out.append((self.ffn(b, step), 1.0))
+        stream.delta = Pending(out)
+        return stream
+
+    __call__ = forward
