@@ -1,0 +1,559 @@
+"""Nevodra through the engine against the plain model (`tests/plain/nevodra.py`, written from the design's equations,
+no cache, float64): every mechanism alone, every way of cutting a prompt, batches, reused pages and slots, window,
+kept-token and page edges, far keys, the sink, the router's choice, long decoding, sizes that are 1 or equal, and
+greedy generation through the engine's own entry point. On the CPU the plain twins of the operations stand in for the
+HIP kernels (this checks configuration, weights, cache, state and batching); the `gpu` cases run the HIP kernels, each
+also alone against its twin."""
+from __future__ import annotations
+
+import functools
+import json
+import pathlib
+
+import pytest
+import torch
+
+from tests import helpers as H
+from tests import nevodra_models as M
+from tests.plain import nevodra as plain
+from tests.plain.ops import TorchKernels
+
+DEVICES = [pytest.param("cpu", id="cpu-twin"), pytest.param("cuda", marks=pytest.mark.gpu, id="hip")]
+DTYPES = ["float32", "bfloat16"]
+MODELS = {"A": (M.CONFIG_A, 11, False, 8), "B": (M.CONFIG_B, 12, False, 16), "C": (M.CONFIG_C, 13, False, 4),
+          "A-sharp": (M.CONFIG_A, 14, True, 16), "B-sharp": (M.CONFIG_B, 15, True, 8), "D-sharp": (M.CONFIG_D, 20, True, 16),
+          "attention": (M.ONLY_ATTENTION, 16, True, 8), "latent": (M.ONLY_LATENT, 17, True, 8),
+          "dense": (M.ONLY_DENSE, 18, False, 8), "moe": (M.ONLY_MOE, 19, False, 8), "filter": (M.ONLY_FILTER, 21, False, 8)}
+LENGTHS = (40, 70, 33, 58, 50, 64, 21)
+# bfloat16 engine against the float64 plain model, relative rms of the logits: what rounding alone gives on these
+# models stays well below this; a lost key, state, sink or expert is far above it on the sharp models.
+BF16_RMS = 0.08
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("nevodra")
+    return {name: M.make_folder(root / name, cfg, seed, sharp) for name, (cfg, seed, sharp, _) in MODELS.items()}
+
+
+@functools.lru_cache(maxsize=None)
+def _plain(folder: str) -> M.PlainNevodra:
+    return M.PlainNevodra(folder)
+
+
+def _requests(name: str, lengths=LENGTHS) -> dict[str, list[int]]:
+    return {f"r{i}": H.random_ids(n, MODELS[name][0]["vocab"], 300 + i) for i, n in enumerate(lengths)}
+
+
+def _replayer(folder, device, dtype, page, cache_tokens, max_seqs=4, max_model_len=256):
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    loaded = load_model(folder, device=device, dtype=dtype, kernels=TorchKernels() if device == "cpu" else None,
+                        page_size=page, max_seqs=max_seqs, max_model_len=max_model_len, max_step_tokens=max_model_len,
+                        cache_tokens=cache_tokens)
+    return Replayer(loaded)
+
+
+def _check(folder, dtype, requests, got, what):
+    folder = pathlib.Path(folder)
+    want = {r: _plain(str(folder)).logits(ids) for r, ids in requests.items()}
+    g, w = H.gather(want, got)
+    assert torch.isfinite(g).all(), f"{what}: non-finite logits"
+    if dtype == "float32":
+        r, m = H.rel_rms(g, w), H.max_over_rms(g, w)
+        assert r <= 3e-5 and m <= 3e-4, f"{what}: float32 logits differ: rms {r:.3g}, max {m:.3g}"
+    else:
+        # In bfloat16 a router's close call may fall the other way (its input is rounded), and the position then has
+        # another expert's output: the float32 runs hold the choice itself, and here the worst 4 % of positions are
+        # set aside for every routed feed-forward a token passes (a repeated layer counts each time). What a lost
+        # key, edge or state does to one position is held by the tests that place it, on models without experts.
+        config = json.loads((folder / "config.json").read_text())
+        routed = sum((config["layers"][i].get("mlp") or {}).get("kind") == "moe" for i, _ in plain.run_order(config))
+        per = (g - w).square().mean(-1).sqrt() / w.square().mean().sqrt()
+        if routed:
+            per = per.sort().values[: len(per) - int(len(per) * min(0.04 * routed, 0.3)) - 1]
+        r = per.square().mean().sqrt().item()
+        assert r <= BF16_RMS, f"{what}: bfloat16 logits differ: rms {r:.3g}"
+        assert per.max().item() <= 3 * BF16_RMS, f"{what}: one position differs by {per.max().item():.3g}"
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(MODELS))
+def test_every_way_of_cutting(folders, name, dtype, device):
+    """Whole prompts (the first tokens of a sequence among them), token-by-token decoding from the second token on and
+    after a long prompt, portions of changing size down to two tokens; in a pool that holds only the longest request,
+    so that every request uses the pages and the slot of the one before."""
+    folder, requests = folders[name], _requests(name)
+    page = MODELS[name][3]
+    rep = _replayer(folder, device, dtype, page, cache_tokens=-(-max(LENGTHS) // page) * page)
+    got = H.run_trace(rep, H.trace_whole({**requests, "one": requests["r0"][:1]}))
+    assert len(got) == sum(LENGTHS) + 1
+    _check(folder, dtype, {**requests, "one": requests["r0"][:1]}, got, f"{name} {dtype} whole")
+    rep.cache.check()
+    for rid, tail in (("r2", len(requests["r2"]) - 1), ("r1", 32)):       # everything after the first token; a tail
+        got = H.run_trace(rep, H.trace_decode_tail(rid, requests[rid], tail))
+        assert len(got) == len(requests[rid])
+        _check(folder, dtype, requests, got, f"{name} {dtype} decode tail {rid}")
+    for rid, sizes in (("r3", [7, 2, 13, 3, 2, 30, 5]), ("r1", [2, 2, 17, 16, 1 + page, 2]), ("r5", [1, 3, page, 2])):
+        got = H.run_trace(rep, H.trace_chunks(rid, requests[rid], sizes))
+        assert len(got) == len(requests[rid])
+        _check(folder, dtype, requests, got, f"{name} {dtype} portions {rid}")
+    rep.cache.check()
+    assert all(g.pool.free == g.pool.usable for g in rep.cache.groups)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B-sharp", "C", "D-sharp"])
+def test_mixed_batches_in_a_small_pool(folders, name, dtype, device):
+    """Unequal requests side by side (portions beside single tokens, requests left out of steps) against each alone;
+    three slots and a pool of the most that is ever live, so that pages and slots are given back and used again."""
+    folder, requests = folders[name], _requests(name)
+    page = MODELS[name][3]
+    for seed in (0, 1):
+        trace = H.trace_mixed(requests, seed=seed, max_live=3, decode_tail=6 + 5 * seed, max_chunk=19)
+        rep = _replayer(folder, device, dtype, page, cache_tokens=H.peak_live_tokens(trace, round_to=page), max_seqs=3)
+        got = H.run_trace(rep, trace)
+        assert len(got) == sum(LENGTHS)
+        _check(folder, dtype, requests, got, f"{name} {dtype} mixed seed {seed}")
+        rep.cache.check()
+        assert all(g.pool.free == g.pool.usable for g in rep.cache.groups)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_float32_does_not_depend_on_the_cut(folders, device):
+    """A position's float32 logits whole, in portions, decoded and in a mixed batch: the same to rounding."""
+    folder, requests = folders["B"], _requests("B", (45, 38, 27))
+    rep = _replayer(folder, device, "float32", 16, cache_tokens=256)
+    whole = H.run_trace(rep, H.trace_whole(requests))
+    cut = H.run_trace(rep, H.trace_chunks("r0", requests["r0"], [3, 2, 16, 5]))
+    tail = H.run_trace(rep, H.trace_decode_tail("r1", requests["r1"], 20))
+    mixed = H.run_trace(rep, H.trace_mixed(requests, seed=5, max_live=3, decode_tail=7))
+    for other in (cut, tail, mixed):
+        for key, row in other.items():
+            assert H.rel_rms(row, whole[key]) < 1e-5, f"{key}: logits depend on how the prompt was cut"
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_the_stream_after_every_layer_run(folders, device):
+    """The residual stream after each run of a layer (a repeated layer counts each time), float32, against the plain
+    model's: the block's pending terms added to its rows."""
+    from holon_amd.engine.batch import StepRow
+    from holon_amd.parts.base import Stream
+    from holon_amd.parts.stream32 import _terms
+    folder = folders["A"]
+    ids = H.random_ids(37, M.CONFIG_A["vocab"], 3)
+    rep = _replayer(folder, device, "float32", 8, cache_tokens=40)
+    slot = rep.cache.admit()
+    rep.cache.reserve(slot, len(ids))
+    step, _ = rep.runner.prepare([StepRow(slot, 0, ids, [])])
+    model = rep.loaded.model
+    stream = Stream(model.embed(step.token_ids, step.token_take))
+    want = _plain(str(folder)).streams(ids)
+    assert len(want) == len(model.sites) == 8
+    for site, ref in zip(model.sites, want):
+        stream = model.blocks[site.layer](stream, step, site)
+        x = stream.h.clone()
+        for term, scale in _terms(stream.delta):
+            x += scale * term.float()
+        assert H.rel_rms(x.cpu(), ref) < 2e-5, f"run {site.run} (layer {site.layer}, pass {site.turn})"
+
+
+def _needle_attention(root, size, keep_first, page):
+    """One attention layer without filter, cap and distance bias (a score depends on the two tokens alone). A pair of
+    token ids (query token, key token) whose score is the largest of all, and a filler token whose scores with them
+    and with itself are lowest, with the queries' norm weight scaled until the pair's weight among a window of fillers
+    is nearly all of it. Returns the folder and the three ids."""
+    cfg = M.model(32, 40, [M.attention(2, 1, 16, 8, 0.25, size=size, keep_first=keep_first)], taps=0)
+    found = {}
+
+    def edit(t):
+        p = {k: v.double() for k, v in t.items()}
+        a_in = plain.rms(p["embed"] * 2.0, 1e-6) * p["l0.norm1"]           # every token's mixer input
+        q = (plain.rms(a_in @ p["l0.mix.q"].T, 1e-6) * p["l0.mix.q.norm"]).view(-1, 2, 16)
+        k = plain.rms(a_in @ p["l0.mix.k"].T, 1e-6) * p["l0.mix.k.norm"]
+        score = torch.einsum("ahd,bd->abh", q, k)[..., 0] * 0.25            # head 0: [query token, key token]
+        a, b = divmod(int(score.argmax()), score.shape[1])
+        filler = int(torch.stack((score[a], score[:, b], score.diagonal())).amax(0).argmin())
+        gain = 9.0 / float(score[a, b] - score[a, filler])                   # the pair stands e^9 above a filler
+        assert gain > 0
+        t["l0.mix.q.norm"] = (p["l0.mix.q.norm"] * gain).bfloat16()
+        t["l0.mix.r1"] = torch.zeros(2).bfloat16()
+        found.update(a=a, b=b, filler=filler)
+    folder = M.make_folder(root, cfg, 77, edit=edit)
+    return folder, found["a"], found["b"], found["filler"]
+
+
+def _both_ways(folder, plain_model, device, dtype, page, cases, what):
+    """`cases`: [(ids, query position)] in pairs (key seen, key not seen). The plain model's logits differ widely
+    within a pair, and the engine follows it in a prompt and when the query is decoded alone."""
+    (ids_in, q_in), (ids_out, q_out) = cases
+    gap = H.rel_rms(plain_model.logits(ids_in)[q_in], plain_model.logits(ids_out)[q_out])
+    assert gap > 0.2, f"{what}: the test's key does not show: {gap}"
+    for ids, at, side in ((ids_in, q_in, "seen"), (ids_out, q_out, "not seen")):
+        rep = _replayer(folder, device, dtype, page, cache_tokens=-(-len(ids) // page) * page, max_model_len=256)
+        got = H.run_trace(rep, H.trace_whole({"p": ids}))
+        _check(folder, dtype, {"p": ids}, got, f"{what} {side}, prompt")
+        assert H.rel_rms(got[("p", at)], plain_model.logits(ids)[at]) < gap / 8
+        got = H.run_trace(rep, H.trace_decode_tail("p", ids, len(ids) - at + 2))
+        _check(folder, dtype, {"p": ids}, got, f"{what} {side}, decoded")
+        assert H.rel_rms(got[("p", at)], plain_model.logits(ids)[at]) < gap / 8, f"{what} {side}, decoded"
+        got = H.run_trace(rep, H.trace_chunks("p", ids, [at - 1, 2, 3]))
+        assert H.rel_rms(got[("p", at)], plain_model.logits(ids)[at]) < gap / 8, f"{what} {side}, a portion of two"
+        rep.cache.check()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("size,page", [(21, 8), (16, 16), (35, 16), (70, 32)])
+def test_a_key_just_inside_and_just_outside_the_window(tmp_path, size, page, dtype, device):
+    """One key whose score stands out, `size - 1` and `size` tokens behind the query, on either side of a page border,
+    behind a kept first token that is a filler."""
+    folder, a, b, filler = _needle_attention(tmp_path / "needle", size, 1, page)
+    plain_model = M.PlainNevodra(folder)
+    for key_at in (page - 1, page, 2 * page + 3):
+        inside = [filler] * key_at + [b] + [filler] * (size - 2) + [a, filler]
+        outside = [filler] * key_at + [b] + [filler] * (size - 1) + [a, filler]
+        _both_ways(folder, plain_model, device, dtype, page, [(inside, key_at + size - 1), (outside, key_at + size)],
+                   f"window {size}, key at {key_at}")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("keep,page", [(1, 8), (5, 8), (8, 8), (17, 16), (70, 16)])
+def test_the_last_kept_token_and_the_first_that_is_not(tmp_path, keep, page, dtype, device):
+    """A window of 10 that keeps the first `keep` tokens: the key whose score stands out as the last kept token and as
+    the one after it, with the query 100 and more tokens later, many windows and freed pages away."""
+    folder, a, b, filler = _needle_attention(tmp_path / "kept", 10, keep, page)
+    plain_model = M.PlainNevodra(folder)
+    n = keep + 100
+    kept = [filler] * (keep - 1) + [b] + [filler] * (n - keep) + [a, filler]
+    gone = [filler] * keep + [b] + [filler] * (n - keep - 1) + [a, filler]
+    _both_ways(folder, plain_model, device, dtype, page, [(kept, n), (gone, n)], f"{keep} kept tokens")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_far_key_and_the_sink_of_the_latent_attention(tmp_path, dtype, device):
+    """Latent attention with the queries' rotated part switched off (a score then depends on the two tokens alone):
+    one key 300 tokens back whose score stands out carries the result across many pages, in a prompt cut into portions
+    and decoded alone; and the sink takes its share: far above the scores it all but silences the mixer."""
+    cfg = M.model(32, 40, [M.latent(2, 16, 4, 8, 12, 0.25)], taps=0)
+    found = {}
+
+    def edit(t, sink=None):
+        p = {k: v.double() for k, v in t.items()}
+        a_in = plain.rms(p["embed"] * 2.0, 1e-6) * p["l0.norm1"]
+        wq = p["l0.mix.q"].view(2, 20, 32).clone()
+        wq[:, 16:] = 0                                                     # no rotated part on the query side
+        q = torch.einsum("tw,hdw->thd", a_in, wq)[..., :16]
+        c = plain.rms((a_in @ p["l0.mix.dkv"].T)[:, :12], 1e-6) * p["l0.mix.dkv.norm"]
+        k = (c @ p["l0.mix.uk"].T).view(-1, 2, 16)
+        score = torch.einsum("ahd,bhd->abh", q, k).amax(-1) * 0.25
+        a, b = divmod(int(score.argmax()), score.shape[1])
+        filler = int(torch.stack((score[a], score[:, b], score.diagonal())).amax(0).argmin())
+        gain = 12.0 / float(score[a, b] - score[a, filler])
+        t["l0.mix.q"] = (wq * gain).reshape(40, 32).bfloat16()
+        t["l0.mix.sink"] = torch.full((2,), -20.0 if sink is None else sink).bfloat16()
+        found.update(a=a, b=b, filler=filler, top=float(score[a, b]) * gain)
+    folder = M.make_folder(tmp_path / "far", cfg, 5, edit=edit)
+    a, b, filler = found["a"], found["b"], found["filler"]
+    plain_model = M.PlainNevodra(folder)
+    ids = [filler] * 3 + [b] + [filler] * 300 + [a, filler]
+    without = [filler] * 304 + [a, filler]
+    at = 304
+    gap = H.rel_rms(plain_model.logits(ids)[at], plain_model.logits(without)[at])
+    assert gap > 0.1, f"the far key does not show: {gap}"
+    rep = _replayer(folder, device, dtype, 16, cache_tokens=320, max_model_len=320)
+    trace = H.trace_chunks("f", ids[:at], [150, 2, 97, 55])
+    trace.steps[-1]["end"] = []
+    trace.add([("f", at, [ids[at]], [0])])
+    trace.add([("f", at + 1, [ids[at + 1]], [0])], end=["f"])
+    got = H.run_trace(rep, trace)
+    _check(folder, dtype, {"f": ids}, got, "far key")
+    assert H.rel_rms(got[("f", at)], plain_model.logits(ids)[at]) < gap / 8
+    got = H.run_trace(rep, H.trace_whole({"f": ids}))
+    assert H.rel_rms(got[("f", at)], plain_model.logits(ids)[at]) < gap / 8
+    sunk = M.make_folder(tmp_path / "sunk", cfg, 5, edit=lambda t: edit(t, sink=found["top"] + 6.0))
+    plain_sunk = M.PlainNevodra(sunk)
+    gap = H.rel_rms(plain_sunk.logits(ids)[at], plain_model.logits(ids)[at])
+    assert gap > 0.1, f"the sink does not show: {gap}"
+    rep = _replayer(sunk, device, dtype, 16, cache_tokens=320, max_model_len=320)
+    got = H.run_trace(rep, H.trace_decode_tail("s", ids, 3))
+    _check(sunk, dtype, {"s": ids}, got, "sink")
+    assert H.rel_rms(got[("s", at)], plain_sunk.logits(ids)[at]) < gap / 8
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_rotation_distance_bias_and_cap_show(folders, tmp_path, device):
+    """The rotated part, the distance bias and the cap each move the plain model's logits far more than the engine
+    differs from it: a mechanism left out or mistaken would not pass the other tests."""
+    ids = H.random_ids(60, 90, 4)
+    for name, key, change in (("latent", "l0.mix.dkv", lambda t: t * 0.0 + t.flip(0)),
+                              ("attention", "l0.mix.r1", lambda t: t * 0.0), ("attention", "l0.mix.r2", lambda t: t * 3.0)):
+        base = _plain(str(folders[name]))
+        cfg, seed, sharp, page = MODELS[name]
+
+        def edit(t, key=key, change=change):
+            t[key] = change(t[key].float()).bfloat16()
+        other = M.PlainNevodra(M.make_folder(tmp_path / f"{name}-{key}", cfg, seed, sharp, edit=edit))
+        gap = H.rel_rms(other.logits(ids), base.logits(ids))
+        rep = _replayer(folders[name], device, "float32", page, cache_tokens=64)
+        got = H.run_trace(rep, H.trace_chunks("x", ids, [23, 2, 9]))
+        g, w = H.gather({"x": base.logits(ids)}, got)
+        assert gap > 1e-2 and H.rel_rms(g, w) < gap / 100, f"{name} {key}: gap {gap}"
+    capped = M.variant(M.ONLY_ATTENTION)
+    base = _plain(str(folders["attention"]))
+    capped["layers"][0]["mixer"]["softcap"] = 400.0
+    other = M.PlainNevodra(M.make_folder(tmp_path / "cap", capped, 16, True))
+    assert H.rel_rms(other.logits(ids), base.logits(ids)) > 1e-2
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_the_router_chooses_as_the_plain_model(device):
+    """The router's weights on their own: groups of neighbours ranked by their two best choice scores, corrections
+    that push choice scores below zero (a closed group must not win with 0), weights from the uncorrected scores."""
+    from holon_amd.kernels.registry import kernel_op
+    import holon_amd.parts  # noqa: F401
+    if device == "cuda":
+        from holon_amd.kernels import load_hip
+        route = load_hip().moe_route
+    else:
+        route = kernel_op("moe_route").plain
+    g = torch.Generator().manual_seed(3)
+    for experts, top, count, keep in ((8, 3, 2, 1), (12, 4, 3, 2), (6, 2, 1, 1), (16, 2, 8, 1), (4, 4, 4, 4), (9, 1, 9, 2)):
+        logits = (2.0 * torch.randn(50, experts, generator=g)).to(device)
+        correction = (torch.randn(experts, generator=g) - 1.5).to(device)       # most choice scores are negative
+        got = route(logits, correction, top, count, keep, 1.7).cpu()
+        router = {"top": top, "scale": 1.7, **({"groups": {"count": count, "keep": keep}} if count > 1 else {})}
+        for t in range(50):
+            s = torch.sigmoid(logits[t].double().cpu())
+            chosen = plain.choose(s, correction.double().cpu(), router)
+            want = torch.zeros(experts, dtype=torch.float64)
+            want[chosen] = 1.7 * s[chosen]
+            assert torch.allclose(got[t].double(), want, atol=1e-6), (experts, top, count, keep, t)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(folders, dtype, device):
+    """180 tokens one by one after a prompt of 5: many window lengths, many pages given back on the way while the
+    kept first tokens' pages stay."""
+    folder, page = folders["A-sharp"], 8
+    ids = H.random_ids(185, M.CONFIG_A["vocab"], 21)
+    rep = _replayer(folder, device, dtype, page, cache_tokens=192)
+    trace = H.trace_decode_tail("d", ids, 180)
+    trace.steps[-1]["end"] = []
+    got = H.run_trace(rep, trace)
+    _check(folder, dtype, {"d": ids}, got, f"long decoding {dtype}")
+    windowed = [g for g in rep.cache.groups if g.decl.window > 0]
+    assert windowed
+    for g in windowed:                             # the window's pages and the kept tokens' pages, no more
+        held = g.pool.usable - g.pool.free
+        assert held <= -(-g.decl.keep_first // page) + -(-g.decl.window // page) + 1, (g.decl, held)
+    rep.cache.check()
+    rep.step([], ["d"])
+    assert all(g.pool.free == g.pool.usable for g in rep.cache.groups)
+
+
+def test_kept_pages_in_the_cache_manager():
+    """A windowed state that keeps its first tokens: their pages stay while the window's are given back, pages of the
+    window that overlap them are not given back twice, and a release returns everything."""
+    from holon_amd.cache.manager import CacheManager
+    from holon_amd.model import Site
+    from holon_amd.parts.base import PagedState
+    sites = [Site(run=0, layer=0), Site(run=1, layer=1)]
+    decls = [[PagedState("kv", 4, window=10, keep_first=5)], [PagedState("kv", 4, window=10, keep_first=0)]]
+    cache = CacheManager(sites, decls, page_size=4, max_seqs=2, max_model_len=64, tokens=64, device=torch.device("cpu"),
+                         dtype=torch.float32)
+    kept, plain_window = cache.groups
+    slot = cache.admit()
+    for total in (3, 9, 20, 21, 40, 64):
+        assert cache.reserve(slot, total)
+        cache.advance(slot, total)
+        cache.check()
+    null = kept.pool.null
+    assert list(kept.table[slot, :2] != null) == [True, True] and (kept.table[slot, 2:13] == null).all()
+    assert (kept.table[slot, 13:16] != null).all() and (plain_window.table[slot, :13] == null).all()
+    assert kept.pool.usable - kept.pool.free == 5 and plain_window.pool.usable - plain_window.pool.free == 3
+    other = cache.admit()
+    assert cache.reserve(other, 40) and cache.could_fit(None, 60, [slot, other]) and not cache.could_fit(None, 60, [other])
+    cache.release(slot)
+    cache.release(other)
+    cache.check()
+    assert all(g.pool.free == g.pool.usable for g in cache.groups)
+
+
+def test_configuration_and_weights_are_checked(tmp_path):
+    from holon_amd.config.model import ConfigError
+    from holon_amd.registry import resolve
+    from holon_amd.weights.loader import WeightError
+    cfg, spec = resolve(M.CONFIG_A)
+    assert [r.layer for r in spec.order] == [0, 1, 2, 1, 2, 1, 2, 3] and cfg.to_dict()["loop"] == M.CONFIG_A["loop"]
+    assert [r.layer for r in resolve(M.CONFIG_C)[1].order] == [0, 1, 2]
+    assert [r.layer for r in resolve(M.CONFIG_D)[1].order] == [0, 1, 0, 1, 2]
+    bad_router = M.variant(M.CONFIG_A)
+    bad_router["layers"][1]["mlp"]["router"]["groups"] = {"count": 3, "keep": 1}
+    bad_rot = M.variant(M.CONFIG_A)
+    bad_rot["layers"][0]["mixer"]["rot"]["dims"] = 10
+    for bad in (M.variant(M.CONFIG_A, loop={"start": 1, "stop": 1, "times": 2}),
+                {k: v for k, v in M.CONFIG_A.items() if k != "norm"},
+                M.variant(M.CONFIG_A, layers=[{"type": "conv", "mixer": {}, "mlp": None}]),
+                M.variant(M.CONFIG_A, layers=[M.attention(3, 2, 8, 8, 1.0)]), bad_router, bad_rot):
+        with pytest.raises(ConfigError):
+            resolve(bad)
+
+    def drop(t):
+        del t["l0.mix.sink"]
+        t["l1.mlp.correction"] = torch.zeros(5).bfloat16()
+    folder = M.make_folder(tmp_path / "bad", M.CONFIG_A, 1, edit=drop)
+    from holon_amd.engine.loading import load_model
+    with pytest.raises(WeightError) as e:
+        load_model(folder, device="cpu", dtype="float32", kernels=TorchKernels(), max_model_len=32, max_seqs=2)
+    assert "l0.mix.sink" in str(e.value) and "l1.mlp.correction" in str(e.value)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_random_weights_from_the_command_line_replay(tmp_path, device):
+    """`holon_amd random` writes a Nevodra folder, and the engine and the plain model agree on it."""
+    from holon_amd.cli import main
+    (tmp_path / "c.json").write_text(json.dumps(M.CONFIG_A))
+    assert main(["random", "--config", str(tmp_path / "c.json"), "--seed", "4", "--out", str(tmp_path / "m")]) == 0
+    ids = H.random_ids(30, M.CONFIG_A["vocab"], 2)
+    rep = _replayer(tmp_path / "m", device, "float32", 8, cache_tokens=32)
+    got = H.run_trace(rep, H.trace_chunks("a", ids, [4, 9]))
+    _check(tmp_path / "m", "float32", {"a": ids}, got, "random folder")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_greedy_generation_through_the_engine(folders, dtype, device):
+    """The engine's own entry point and scheduler: prompts of unequal length generated side by side, with prompt
+    portions riding beside decode rows, follow the plain model's most likely token wherever that is clear."""
+    from holon_amd.config import EngineConfig, SamplingParams
+    from holon_amd.engine.engine import Engine
+    folder = folders["B-sharp"]
+    plain_model = _plain(str(folder))
+    prompts = [H.random_ids(n, M.CONFIG_B["vocab"], 50 + n) for n in (5, 37, 18, 1)]
+    cfg = EngineConfig(model=str(folder), device=device, dtype=dtype, page_size=8, max_seqs=3, max_model_len=96,
+                       max_step_tokens=40, chunk_with_decode=16, cache_tokens=192)
+    engine = Engine(cfg, TorchKernels() if device == "cpu" else None)
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True))
+    held = sum(H.assert_greedy_follows(plain_model, p, o, margin=0.02 if dtype == "float32" else 0.25)
+               for p, o in zip(prompts, outs))
+    assert all(len(o) == 24 for o in outs) and held >= (60 if dtype == "float32" else 20)
+    engine.cache.check()
+    engine.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,dtype", [("A-sharp", "float32"), ("A-sharp", "bfloat16"), ("D-sharp", "float32")])
+def test_graph_replays_equal_eager_steps(folders, name, dtype):
+    """Decode steps replayed from HIP graphs give the tokens of eager steps, over many replays with the program's own
+    eager work (prompt steps, sampling, host synchronisation) between them, while the batch shrinks through the
+    buckets, pages are taken and given back and windows pass."""
+    from holon_amd.config import EngineConfig, SamplingParams
+    from holon_amd.engine.engine import Engine
+    vocab = MODELS[name][0]["vocab"]
+    prompts = [H.random_ids(n, vocab, 80 + n) for n in (3, 17, 8, 25, 40, 1)]
+    outs = {}
+    for graphs in (False, True):
+        engine = Engine(EngineConfig(model=str(folders[name]), device="cuda", dtype=dtype, page_size=16, max_seqs=6,
+                                     max_model_len=160, max_step_tokens=64, graphs=graphs, cache_tokens=960))
+        rids = [engine.add(p, SamplingParams(temperature=0.0 if i % 2 else 0.7, seed=5, max_tokens=60 + 7 * i,
+                                             ignore_eos=True)) for i, p in enumerate(prompts)]
+        got = {r: [] for r in rids}
+        while engine.has_work():
+            for d in engine.step():
+                got[d.rid].extend(d.token_ids)
+        outs[graphs] = [got[r] for r in rids]
+        engine.cache.check()
+        if graphs:
+            assert engine.runner.graph_replays > 20 and len(engine.runner.graphs) >= 3
+        engine.close()
+    assert outs[True] == outs[False]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_kernels_alone_against_their_plain_forms(dtype):
+    """Every operation the design brought, on the GPU, against its plain form in torch: odd widths, rows wider than a
+    block holds in registers, windows with and without kept tokens over scattered pages."""
+    import holon_amd.parts  # noqa: F401
+    from holon_amd.kernels import load_hip
+    from holon_amd.kernels.registry import kernel_op
+    from holon_amd.parts.positions import rope_table
+    k, dev = load_hip(), "cuda"
+    tol = 2e-6 if dtype == torch.float32 else 6e-3
+    g = torch.Generator().manual_seed(0)
+
+    def randn(*shape, to=dtype):
+        return torch.randn(*shape, generator=g).to(dev).to(to)
+    for dim in (96, 250, 1500, 5000):
+        x, t1, t2 = randn(7, dim, to=torch.float32), randn(7, dim), randn(7, dim)
+        row, w1, w2 = randn(dim, to=torch.float32), randn(dim), randn(dim)
+        xa, xb = x.clone(), x.clone()
+        a = k.stream_rms(xa, [(t1, 1.0), (t2, 1.0)], row, w1, w2, 1e-6, dtype)
+        b = kernel_op("stream_rms").plain(xb, [(t1, 1.0), (t2, 1.0)], row, w1, w2, 1e-6, dtype)
+        assert H.rel_rms(xa, xb) < 1e-6 and H.rel_rms(a[0], b[0]) < tol and H.rel_rms(a[1], b[1]) < tol, dim
+    for dim in (80, 321, 3000, 9000):
+        z, coef = randn(5, dim), torch.tensor([0.5, -0.3, 0.2, 0.1], device=dev)
+        assert H.rel_rms(k.polynorm(z, coef, 1e-6), kernel_op("polynorm").plain(z, coef, 1e-6)) < tol, dim
+    experts, ff, shared = 6, 24, 40
+    gate_up = randn(9, 2 * (experts * ff + shared))
+    weights = kernel_op("moe_route").plain(randn(9, experts, to=torch.float32), None, 2, 1, 1, 1.5)
+    assert H.rel_rms(k.moe_gate(gate_up, weights, ff, shared), kernel_op("moe_gate").plain(gate_up, weights, ff, shared)) < tol
+    x = randn(5, 77)
+    assert torch.equal(k.scale_rows(x, 3.0), x.float() * 3.0)
+    # a paged cache of three rows over scattered pages
+    page, heads, groups, dim, vdim, n_pages = 16, 4, 2, 24, 40, 40
+    lens = [70, 33, 150]
+    table = torch.full((4, 12), n_pages - 1, dtype=torch.int32)
+    order, at = torch.randperm(n_pages - 1, generator=g).tolist(), 0
+    for s, n in enumerate(lens):
+        for i in range(-(-n // page)):
+            table[s, i] = order[at]
+            at += 1
+    table = table.to(dev)
+    token_row = torch.cat([torch.full((n,), i, dtype=torch.int32) for i, n in enumerate(lens)]).to(dev)
+    positions = torch.cat([torch.arange(n, dtype=torch.int32) for n in lens]).to(dev)
+    write_page = table[token_row.long(), (positions // page).long()].contiguous()
+    write_off = (positions % page).to(torch.int32)
+    total = sum(lens)
+    qkv = randn(total, (heads + groups) * dim + groups * vdim)
+    qw, kw = (1 + 0.2 * randn(heads * dim, to=torch.float32)).to(dtype), (1 + 0.2 * randn(groups * dim, to=torch.float32)).to(dtype)
+    pages_a = torch.zeros(n_pages, groups * page * (dim + vdim), device=dev, dtype=dtype)
+    pages_b = pages_a.clone()
+    qa = k.whole_norm_prepare(qkv, heads, groups, dim, vdim, qw, kw, 1e-6, pages_a, write_page, write_off, page)
+    qb = kernel_op("whole_norm_prepare").plain(qkv, heads, groups, dim, vdim, qw, kw, 1e-6, pages_b, write_page,
+                                               write_off, page)
+    assert H.rel_rms(qa, qb) < tol and H.rel_rms(pages_a, pages_b) < tol
+
+    class Rows:
+        slots = torch.tensor([0, 1, 2], dtype=torch.int32, device=dev)
+    r1, r2 = torch.rand(heads, generator=g).to(dev), (2 * torch.rand(heads, generator=g)).to(dev)
+    sink = randn(heads, to=torch.float32)
+    q = (qb.float() * 3).to(dtype)
+    for window, keep, cap, dist, sk in ((0, 0, 0.0, None, None), (20, 0, 0.0, None, sink), (40, 5, 3.0, (r1, r2), None),
+                                        (17, 20, 0.0, (r1, r2), sink), (64, 70, 5.0, None, None), (3, 1, 0.0, None, None),
+                                        (100, 64, 2.0, (r1, r2), None), (1, 65, 0.0, None, None)):
+        args = (q, pages_b, table, Rows, token_row, positions, groups, vdim, page, sk, 0.3, window)
+        a = k.softmax_attention(*args, softcap=cap, dist=dist, keep_first=keep)
+        b = kernel_op("softmax_attention").plain(*args, softcap=cap, dist=dist, keep_first=keep)
+        assert H.rel_rms(a, b) < tol, (window, keep, cap)
+    h2, dm, rot, rank, rd = 3, 16, 8, 24, 6
+    tab = rope_table(256, rd, 1000.0).to(dev)
+    both = randn(total, h2 * (dm + rot) + rank + rot)
+    cw = (1 + 0.2 * randn(rank, to=torch.float32)).to(dtype)
+    pa = torch.zeros(n_pages, 2 * page * (rank + rot), device=dev, dtype=dtype)
+    pb = pa.clone()
+    a = k.latent_rope_prepare(both, h2, dm, rot, rank, cw, 1e-6, tab, positions, pa, write_page, write_off, page)
+    b = kernel_op("latent_rope_prepare").plain(both, h2, dm, rot, rank, cw, 1e-6, tab, positions, pb, write_page,
+                                               write_off, page)
+    assert H.rel_rms(a[0], b[0]) < tol and H.rel_rms(a[1][..., rank:], b[1][..., rank:]) < tol and H.rel_rms(pa, pb) < tol
+    for t in (5, 40):
+        x, w = randn(t, h2, dm), randn(h2, rank, dm)
+        full = torch.zeros(t, h2, rank + rot, device=dev, dtype=dtype)
+        k.head_linear(x, w, out=full[..., :rank])
+        assert H.rel_rms(full[..., :rank], kernel_op("head_linear").plain(x, w)) < tol and not full[..., rank:].any()
