@@ -21,7 +21,7 @@ The engine is one process on one GPU; for --gpus > 1 a line says so and the exit
 prompt tokens at the Qwen3-32B shape, portions of 512 tokens beside decode rows, 256 greedy tokens each; `long` is 8
 prompts of 32,768 tokens at the Qwen3-4B shape, 512 tokens each at temperature 0.7.
 
---workload tolurax (or relanex) measures that design beside Qwen3 at equal sizes (width, layers, heads, head size,
+--workload tolurax (or relanex, or nevodra) measures that design beside Qwen3 at equal sizes (width, layers, heads, head size,
 feed-forward, vocabulary; random weights): a 2,048-token prompt and decode at batch 8 near a context of 2,048, at two
 sizes (`--sizes`), one line with both models' figures and the bytes a decode step must read. `--only` runs one model
 (for a profiler).
@@ -146,6 +146,29 @@ def relanex_config(z: dict, window: int = 1024) -> dict:
             "residual_mult": 0.5, "layers": [layer(i) for i in range(z["layers"])]}
 
 
+def nevodra_config(z: dict, window: int = 1024) -> dict:
+    """A Nevodra model of a size's layers, in pairs: windowed attention with the size's heads (a tanh cap, a distance
+    bias, four kept first tokens) over a dense PolyNorm feed-forward of the size's width, then latent attention (the
+    size's heads, a latent of 192 and 64 rotated dimensions: cache entries of 256) over eight experts of a quarter of
+    that width of which a token uses two, beside a shared one; filters of three taps on every sublayer's input."""
+    def layer(i: int) -> dict:
+        if i % 2 == 0:
+            return {"type": "attention", "mlp": {"kind": "dense", "ff": z["ff"]},
+                    "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                              "scale": z["dim"] ** -0.5, "softcap": 30.0, "mask": {"size": window, "keep_first": 4}}}
+        quarter = z["ff"] // 4
+        return {"type": "latent_attention",
+                "mlp": {"kind": "moe", "expert": {"ff": quarter}, "shared": {"ff": quarter},
+                        "router": {"experts": 8, "top": 2, "scale": 1.5, "groups": {"count": 4, "keep": 2}}},
+                "mixer": {"heads": z["heads"], "dim": z["dim"], "rot_dim": 64, "vdim": z["dim"], "kv_rank": 192,
+                          "scale": (z["dim"] + 64) ** -0.5, "rot": {"dims": 64, "base": 1e6}}}
+    return {"architecture": "Nevodra", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "canon": {"taps": 3}, "layers": [layer(i) for i in range(z["layers"])]}
+
+
+DESIGN_CONFIGS = {"tolurax": tolurax_config, "relanex": relanex_config, "nevodra": nevodra_config}
+
+
 def design_cache_bytes(name: str, cfg_json: dict, z: dict, item: int, batch: int, context: int) -> int:
     """The bytes of paged cache a decode step of `batch` rows near `context` reads."""
     if name == "qwen3":
@@ -156,9 +179,11 @@ def design_cache_bytes(name: str, cfg_json: dict, z: dict, item: int, batch: int
         if layer["type"] == "parallel":             # the window's keys and values
             total += 2 * z["kv_heads"] * z["dim"] * item * batch * min(context, m["left"]["mask"]["size"])
         elif layer["type"] == "attention":
-            total += m["kv_heads"] * (m["dim"] + m["vdim"]) * item * batch * context
-        elif layer["type"] == "latent_attention":   # the latent, held as keys and as values
-            total += 2 * m["kv_rank"] * item * batch * min(context, m["mask"]["size"])
+            seen = min(context, m["mask"]["size"] + m["mask"].get("keep_first", 0)) if m.get("mask") else context
+            total += m["kv_heads"] * (m["dim"] + m["vdim"]) * item * batch * seen
+        elif layer["type"] == "latent_attention":   # the cache entry, held as keys and as values
+            seen = min(context, m["mask"]["size"]) if m.get("mask") else context
+            total += 2 * (m["kv_rank"] + m.get("rot_dim", 0)) * item * batch * seen
     return total
 
 
@@ -183,7 +208,7 @@ def design(a) -> int:
     out: dict = {}
     for size in a.sizes.split(","):
         z = DESIGN_SIZES[size]
-        ours = tolurax_config(z) if a.workload == "tolurax" else relanex_config(z)
+        ours = DESIGN_CONFIGS[a.workload](z)
         for name, cfg_json in ((a.workload, ours), ("qwen3", qwen3_config(z))):
             if a.only and a.only != name:
                 continue
@@ -256,10 +281,10 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--context", type=int, default=CONTEXT, help="the context the timed decode steps end at")
     ap.add_argument("--prompt", type=int, default=PROMPT, help="tokens of the timed prompt")
     ap.add_argument("--no-graphs", action="store_true")
-    ap.add_argument("--workload", choices=("decode", "mixed", "long", "tolurax", "relanex"), default="decode")
-    ap.add_argument("--sizes", default="2k,4k", help="--workload tolurax|relanex: which of its sizes (2k, 4k) to run")
-    ap.add_argument("--only", choices=("tolurax", "relanex", "qwen3"), default=None,
-                    help="--workload tolurax|relanex: one model only")
+    ap.add_argument("--workload", choices=("decode", "mixed", "long", "tolurax", "relanex", "nevodra"), default="decode")
+    ap.add_argument("--sizes", default="2k,4k", help="--workload tolurax|relanex|nevodra: which of its sizes (2k, 4k) to run")
+    ap.add_argument("--only", choices=("tolurax", "relanex", "nevodra", "qwen3"), default=None,
+                    help="--workload tolurax|relanex|nevodra: one model only")
     ap.add_argument("--products", choices=("own", "vendor", "timed"), default="timed",
                     help="EngineConfig.products: which kernel products of 17 to 1,024 rows take (reported in the line)")
     a = ap.parse_args(argv)
@@ -270,7 +295,7 @@ def main(argv: list[str] | None = None) -> int:
         from .kernels import build as kernel_build
         if kernel_build.find_library() is None:
             kernel_build.build()
-        if a.workload in ("tolurax", "relanex"):
+        if a.workload in DESIGN_CONFIGS:
             return design(a)
         return workload(a.workload, None if "--layers" not in (argv or sys.argv) else a.layers, a.dtype, a.products)
 
