@@ -65,6 +65,18 @@ struct AttnArgs {
   // softmax with a sink (nullable, [Hq], in the scores' natural units): exp(sink[head] - max) joins the denominator;
   // it has no key and no value
   const float* sink;
+  // changed scores (the kernels instantiated with MOD only; `scale` above is then the scores' scale): s <- softcap
+  // tanh(s / softcap) where softcap > 0; then s <- s - r1[head] ln(1 + r2[head] (i - j)) for query i and key j where r1
+  // is given; and under a window, keys 0 .. keep_first - 1 stay visible to every query behind them
+  float softcap;
+  const float* r1;
+  const float* r2;
+  int keep_first;
+};
+
+// What a lane needs to change its column's scores: the head's two numbers of the distance bias.
+struct ModLane {
+  float b1, b2;
 };
 
 // The denominator of a row whose keys summed to `l` under the running maximum `m` (in units of log2): with a sink, its
@@ -92,20 +104,38 @@ __host__ __device__ inline TileMap tile_map(int group) {
 // running max and sum, the probabilities as the next product's B operand, and the rescale of what was summed so far
 // (only when some row's max moved: later blocks rarely move it, and the accumulators can then stay where the matrix
 // cores keep them). Lane (g, c): s0[r] is key kb+8g+r against query column c, s1[r] key kb+8g+4+r.
-template <int DS>
+// MOD: the scores are changed first (see AttnArgs: scale, cap, distance bias, in natural units; they then enter the
+// exponential times log2(e)), and keys below `keep_first` are seen whatever the window says.
+template <int DS, bool MOD = false>
 __device__ __forceinline__ bf16x8_t softmax_block(const f32x4_t& s0, const f32x4_t& s1, bool whole, int kb, int g,
                                                   int qp, int first, int key_lo, int key_hi, float scale_log2,
-                                                  float& m, float& l, f32x4_t (&o)[DS]) {
+                                                  float& m, float& l, f32x4_t (&o)[DS], float mod_scale = 0.f,
+                                                  float softcap = 0.f, ModLane md = ModLane{0.f, 0.f},
+                                                  int keep_first = 0) {
   // m and the comparisons are in units of the raw scores' scale times log2(e); a score enters as one fused
   // multiply-add, exp2(s * c - m)
   float sv[8];
 #pragma unroll
   for (int r = 0; r < 8; ++r) sv[r] = r < 4 ? s0[r] : s1[r - 4];
+  if constexpr (MOD) {
+    const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      float v = sv[r] * mod_scale;
+      if (softcap > 0.f)       // cap tanh(v / cap), tanh(x) = 1 - 2 / (1 + e^(2x))
+        v = softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * v * inv_cap)));
+      const int dist = max(qp - (kb + 8 * g + r), 0);
+      v -= md.b1 * __logf(1.0f + md.b2 * (float)dist);
+      sv[r] = v;
+    }
+    scale_log2 = 1.4426950408889634f;
+  }
   if (!whole) {
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       const int key = kb + 8 * g + r;
-      if (!(key <= qp && key >= first && key >= key_lo && key <= key_hi)) sv[r] = -INFINITY;
+      const bool seen = key <= qp && key <= key_hi && ((key >= first && key >= key_lo) || (MOD && key < keep_first));
+      if (!seen) sv[r] = -INFINITY;
     }
   }
   float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
@@ -165,14 +195,17 @@ struct Nothing {
   __device__ __forceinline__ void operator()() const {}
 };
 // SIG: sigmoid weights (`sig_bias[t]`: the bias of this lane's column in tile t); m and l are then left as they are.
-template <int D, int NT, typename Prepare = Nothing, bool SIG = false>
+// MOD: changed scores (`mod[t]`: the distance bias of this lane's column in tile t), and `kept_keys` > 0: keys
+// 0 .. kept_keys - 1 are walked as well, in blocks of their own in front of key_lo's where they lie before it.
+template <int D, int NT, typename Prepare = Nothing, bool SIG = false, bool MOD = false>
 __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __restrict__ trow, int hk,
                                            const bf16x8_t (&qf)[NT][D / 32], const int (&qpos)[NT],
                                            const int (&tile_last)[NT], const int (&tile_first)[NT], int key_lo,
                                            int key_hi,
                                            f32x4_t (&o)[NT][D / 16], float (&m)[NT], float (&l)[NT],
                                            const bf16_t* fresh = nullptr, Prepare prepare = Prepare(),
-                                           const float* sig_bias = nullptr) {
+                                           const float* sig_bias = nullptr, const ModLane* mod = nullptr,
+                                           int kept_keys = 0) {
   const int lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
   const int P = a.page_size;
@@ -204,13 +237,17 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
     }
   };
   const int kb_first = (key_lo / 32) * 32;
+  // the blocks of kept keys that lie wholly before key_lo's block come first: 0, 32, .. below kept_end, then kb_first on
+  const int kept_end = MOD ? min((kept_keys + 31) / 32 * 32, kb_first) : 0;
+  auto after = [&](int kb) { return MOD && kb + 32 == kept_end ? kb_first : kb + 32; };
+  const int kb_start = kept_end > 0 ? 0 : kb_first;
   int e_cur[2], e_next[2];
-  lookup(kb_first, e_cur);
-  lookup(kb_first + 32, e_next);
+  lookup(kb_start, e_cur);
+  lookup(after(kb_start), e_next);
   bf16x8_t kf0[D / 32], kf1[D / 32];
-  load_keys(kb_first, e_cur, kf0, kf1);
+  load_keys(kb_start, e_cur, kf0, kf1);
   prepare();
-  for (int kb = kb_first; kb <= key_hi; kb += 32) {
+  for (int kb = kb_start; kb <= key_hi; kb = after(kb)) {
     // values of this block (lane group g needs keys 8g .. 8g+7, for dims dsub*16 + c) and the keys of the next one
     // are requested before this block's products, so that their latency hides behind the matrix cores
     const int vkey = kb + (g >= 2 ? 16 : 0);
@@ -222,6 +259,10 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
     if (kb + 31 > key_hi) {
 #pragma unroll
       for (int ds = 0; ds < D / 16; ++ds) zero_after(vf[ds], kb + 8 * g, key_hi);
+    }
+    if (MOD && kb < kept_end) {                            // a kept block: what lies behind the kept keys is not held
+#pragma unroll
+      for (int ds = 0; ds < D / 16; ++ds) zero_after(vf[ds], kb + 8 * g, kept_keys - 1);
     }
     if (fresh != nullptr && kb + 31 >= key_hi) {           // the block that holds key_hi: its key and value from LDS
       const int k0 = kb + 16 * khalf + kin;                // this lane's keys are k0 and k0 + 4
@@ -244,11 +285,12 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
       }
     }
     bf16x8_t nf0[D / 32], nf1[D / 32];
-    const bool more = kb + 32 <= key_hi;
+    const int kb_next = after(kb);
+    const bool more = kb_next <= key_hi;
     int e_after[2] = {0, 0};
     if (more) {
-      load_keys(kb + 32, e_next, nf0, nf1);
-      lookup(kb + 64, e_after);                  // (an entry past the row's keys is clamped into the table and unused)
+      load_keys(kb_next, e_next, nf0, nf1);
+      lookup(after(kb_next), e_after);           // (an entry past the row's keys is clamped into the table and unused)
     }
     bf16x8_t pb[NT], pl[NT];
 #pragma unroll
@@ -266,6 +308,9 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
                          (a.window <= 0 || kb >= tile_last[t] - a.window + 1);
       if constexpr (SIG)
         sigmoid_block(s0, s1, whole, kb, g, qp, first, key_lo, key_hi, a.scale, sig_bias[t], pb[t], pl[t]);
+      else if constexpr (MOD)
+        pb[t] = softmax_block<D / 16, true>(s0, s1, whole, kb, g, qp, first, key_lo, key_hi, a.scale_log2, m[t], l[t],
+                                            o[t], a.scale, a.softcap, mod[t], a.window > 0 ? a.keep_first : 0);
       else
         pb[t] = softmax_block<D / 16>(s0, s1, whole, kb, g, qp, first, key_lo, key_hi, a.scale_log2, m[t], l[t], o[t]);
     }
@@ -307,7 +352,7 @@ __device__ __forceinline__ RowRef row_ref(const TileMap& tm, int c, int p0, int 
   return r;
 }
 
-template <int D, int NT>
+template <int D, int NT, bool MOD = false>
 __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int g = lane / 16, c = lane % 16;
@@ -359,7 +404,17 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
 #pragma unroll
     for (int ds = 0; ds < D / 16; ++ds) o[t][ds] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
-  attn_tiles<D, NT>(a, trow, hk, qf, qpos, tile_last, tile_first, key_lo, key_hi, o, m, l);
+  if constexpr (MOD) {
+    ModLane mod[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      mod[t] = rr[t].valid && a.r1 ? ModLane{a.r1[rr[t].head], a.r2[rr[t].head]} : ModLane{0.f, 0.f};
+    attn_tiles<D, NT, Nothing, false, true>(a, trow, hk, qf, qpos, tile_last, tile_first, key_lo, key_hi, o, m, l,
+                                            nullptr, Nothing(), nullptr, mod,
+                                            a.window > 0 ? min(a.keep_first, key_lo) : 0);
+  } else {
+    attn_tiles<D, NT>(a, trow, hk, qf, qpos, tile_last, tile_first, key_lo, key_hi, o, m, l);
+  }
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     float lt = l[t];
@@ -1505,7 +1560,8 @@ struct NewKeyValue {
 // itself and no merge kernel follows.
 // SIG: sigmoid weights (see AttnArgs): the waves' partials are plain sums (their maxima stay 0, so the combination above
 // adds them as they are), one block a (row, kv head) writes the result, multiplied by the gate's sigmoid if one is given.
-template <int D, bool FUSED, bool SIG = false>
+// MOD: changed scores (see AttnArgs); the wave that takes the row's first share also walks the kept first keys.
+template <int D, bool FUSED, bool SIG = false, bool MOD = false>
 __global__ void __launch_bounds__(512) attn_decode_kernel(AttnArgs a, FusedArgs f) {
   extern __shared__ __attribute__((aligned(16))) float red[];   // [waves - 1][16 D values, 16 maxima, 16 sums]
   __shared__ __attribute__((aligned(16))) bf16_t fresh_lds[FUSED ? 2 * D : 8];
@@ -1624,8 +1680,17 @@ __global__ void __launch_bounds__(512) attn_decode_kernel(AttnArgs a, FusedArgs 
     };
     int qpos[1] = {rr.valid ? qp_row : -1}, tile_last[1] = {qp_row}, tile_first[1] = {qp_row};
     const float sig_bias[1] = {SIG && rr.valid && a.head_bias ? a.head_bias[rr.head] : 0.f};
-    attn_tiles<D, 1, decltype(make_queries), SIG>(a, trow, hk, qf, qpos, tile_last, tile_first, max(key_lo, first),
-                                                  key_hi, o, m, l, writer ? fresh_lds : nullptr, make_queries, sig_bias);
+    if constexpr (MOD) {
+      const ModLane mod[1] = {rr.valid && a.r1 ? ModLane{a.r1[rr.head], a.r2[rr.head]} : ModLane{0.f, 0.f}};
+      attn_tiles<D, 1, decltype(make_queries), false, true>(a, trow, hk, qf, qpos, tile_last, tile_first,
+                                                            max(key_lo, first), key_hi, o, m, l, nullptr, make_queries,
+                                                            nullptr, mod,
+                                                            split == 0 && a.window > 0 ? min(a.keep_first, first) : 0);
+    } else {
+      attn_tiles<D, 1, decltype(make_queries), SIG>(a, trow, hk, qf, qpos, tile_last, tile_first, max(key_lo, first),
+                                                    key_hi, o, m, l, writer ? fresh_lds : nullptr, make_queries,
+                                                    sig_bias);
+    }
   }
   float lt = l[0];
   lt += __shfl_xor(lt, 16, WAVE);
@@ -1794,10 +1859,18 @@ extern "C" int holon_attention_mfma_supported(int head_dim, int page_size, int d
   return dtype == HOLON_BF16 && mfma_serves(head_dim, page_size);
 }
 
+// Changed scores, from the host: see AttnArgs.
+struct ScoreMod {
+  float softcap;
+  const float* r1;
+  const float* r2;
+  int keep_first;
+};
+
 static int prefill_launch(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
                           const int32_t* slots, const int32_t* lens, const int32_t* query_start, const int32_t* row_ids,
                           int n_rows, int max_query, int max_len, int heads, int kv_heads, int head_dim, int page_size,
-                          float scale, int window, const float* sink, void* stream) {
+                          float scale, int window, const float* sink, void* stream, const ScoreMod* mod = nullptr) {
   HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
@@ -1809,8 +1882,24 @@ static int prefill_launch(const void* q, void* out, const void* pages, const int
   a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size;
   a.scale_log2 = scale * 1.4426950408889634f; a.window = window; a.sink = sink;
   const TileMap tm = tile_map(heads / kv_heads);
-  const int nt = head_dim == 256 ? 1 : 2;
   const int tiles = (max_query + tm.pos_per_tile - 1) / tm.pos_per_tile;
+  if (mod != nullptr) {
+    // changed scores: the kernel that reads its operands from the cache, one tile a wave under a window (a wave then
+    // walks its own tile's window and no other's), two without
+    HOLON_CHECK(mod->softcap >= 0.f && mod->keep_first >= 0 && (mod->r1 == nullptr) == (mod->r2 == nullptr),
+                "attention: a cap of %g, %d kept tokens, a distance bias of two numbers a head", mod->softcap,
+                mod->keep_first);
+    a.scale = scale; a.softcap = mod->softcap; a.r1 = mod->r1; a.r2 = mod->r2; a.keep_first = mod->keep_first;
+    const int mnt = head_dim == 256 || window > 0 ? 1 : 2;
+    dim3 grid(((tiles + mnt - 1) / mnt + 3) / 4, kv_heads * tm.head_blocks, n_rows);
+    hipStream_t ms = (hipStream_t)stream;
+    if (head_dim == 64) { if (mnt == 1) attn_prefill_kernel<64, 1, true><<<grid, 256, 0, ms>>>(a); else attn_prefill_kernel<64, 2, true><<<grid, 256, 0, ms>>>(a); }
+    else if (head_dim == 128) { if (mnt == 1) attn_prefill_kernel<128, 1, true><<<grid, 256, 0, ms>>>(a); else attn_prefill_kernel<128, 2, true><<<grid, 256, 0, ms>>>(a); }
+    else attn_prefill_kernel<256, 1, true><<<grid, 256, 0, ms>>>(a);
+    HOLON_LAUNCH_OK();
+    return 0;
+  }
+  const int nt = head_dim == 256 ? 1 : 2;
   if (head_dim != 256 && tiles >= 16 && max_len <= 4096 * page_size) {
     // long portions: keys and values staged through LDS, shared by four waves (rows of up to 4096 pages). Two tiles a
     // wave share each stage among twice the rows (measured: 4,096 tokens 340 -> 287 us, 32,768 tokens 17.0 -> 13.3 ms)
@@ -1950,7 +2039,7 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
                          int n_rows, int max_len, int heads, int kv_heads, int head_dim, int page_size, float scale,
                          int window, float* part_o, float* part_ml, int splits, int keys_per_split, void* stream,
                          const FusedArgs* fused = nullptr, int waves = 1, int rows_in_order = 0,
-                         const float* sink = nullptr) {
+                         const float* sink = nullptr, const ScoreMod* mod = nullptr) {
   HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
@@ -1979,7 +2068,16 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
   hipStream_t s = (hipStream_t)stream;
   const int threads = waves * WAVE;
   const size_t lds = (size_t)(waves - 1) * (16 * head_dim + 32) * sizeof(float);
-  if (fused != nullptr) {
+  if (mod != nullptr) {
+    HOLON_CHECK(fused == nullptr && mod->softcap >= 0.f && mod->keep_first >= 0 && (mod->r1 == nullptr) == (mod->r2 == nullptr),
+                "attention decode: a cap of %g, %d kept tokens, a distance bias of two numbers a head", mod->softcap,
+                mod->keep_first);
+    a.scale = scale; a.softcap = mod->softcap; a.r1 = mod->r1; a.r2 = mod->r2; a.keep_first = mod->keep_first;
+    const FusedArgs none{};
+    if (head_dim == 64) attn_decode_kernel<64, false, false, true><<<grid, threads, lds, s>>>(a, none);
+    else if (head_dim == 128) attn_decode_kernel<128, false, false, true><<<grid, threads, lds, s>>>(a, none);
+    else attn_decode_kernel<256, false, false, true><<<grid, threads, lds, s>>>(a, none);
+  } else if (fused != nullptr) {
     if (head_dim == 64) attn_decode_kernel<64, true><<<grid, threads, lds, s>>>(a, *fused);
     else if (head_dim == 128) attn_decode_kernel<128, true><<<grid, threads, lds, s>>>(a, *fused);
     else attn_decode_kernel<256, true><<<grid, threads, lds, s>>>(a, *fused);
@@ -2039,6 +2137,34 @@ extern "C" int holon_attention_decode_sink_bf16(const void* q, void* out, const 
   return decode_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len, heads,
                        kv_heads, head_dim, page_size, scale, window, part_o, part_ml, splits, keys_per_split, stream,
                        nullptr, waves, rows_in_order, sink);
+}
+
+// The same with changed scores (see AttnArgs): a tanh cap (0: none), a distance bias of two numbers a head (null: none)
+// and, under a window, `keep_first` first keys that stay visible.
+extern "C" int holon_attention_decode_mod_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                               int table_stride, const int32_t* slots, const int32_t* lens,
+                                               const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                               int max_len, int heads, int kv_heads, int head_dim, int page_size,
+                                               float scale, int window, float* part_o, float* part_ml, int splits,
+                                               int keys_per_split, int waves, int rows_in_order, const float* sink,
+                                               float softcap, const float* r1, const float* r2, int keep_first,
+                                               void* stream) {
+  const ScoreMod mod{softcap, r1, r2, keep_first};
+  return decode_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len, heads,
+                       kv_heads, head_dim, page_size, scale, window, part_o, part_ml, splits, keys_per_split, stream,
+                       nullptr, waves, rows_in_order, sink, &mod);
+}
+
+extern "C" int holon_attention_prefill_mod_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                                int table_stride, const int32_t* slots, const int32_t* lens,
+                                                const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                                int max_query, int max_len, int heads, int kv_heads, int head_dim,
+                                                int page_size, float scale, int window, const float* sink,
+                                                float softcap, const float* r1, const float* r2, int keep_first,
+                                                void* stream) {
+  const ScoreMod mod{softcap, r1, r2, keep_first};
+  return prefill_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_query, max_len,
+                        heads, kv_heads, head_dim, page_size, scale, window, sink, stream, &mod);
 }
 
 // Decode rows straight from the step's raw q/k/v projection: per-head norm, rotation and the cache write of each

@@ -19,46 +19,113 @@ __device__ __forceinline__ void block_sum3_256(float& a, float& b, float& c, flo
   c = (part[2][0] + part[2][1]) + (part[2][2] + part[2][3]);
 }
 
-// One block a row: y = a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over the row.
-template <typename T, int REGS>
+// One block a row: y = a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over the row. A thread takes
+// N neighbouring values at a time (N = 16 bytes' worth where rows allow, else 1); REGS such groups stay in registers
+// between the two passes (0: the row is read again).
+template <typename T, int REGS, bool VEC>
 __global__ void __launch_bounds__(256) polynorm_kernel(const T* __restrict__ z, const float* __restrict__ coef,
                                                        T* __restrict__ y, int dim, float eps) {
   __shared__ float part[3][4];
+  constexpr int N = VEC ? Elem<T>::kVec : 1;
   const int64_t base = (int64_t)blockIdx.x * dim;
-  float held[REGS > 0 ? REGS : 1];
+  float held[(REGS > 0 ? REGS : 1) * N];
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
   auto take = [&](float v) { const float q = v * v; s2 += q; s4 += q * q; s6 += q * q * q; };
+  auto load = [&](int i, float* to) {                    // N values from column i on
+    if constexpr (VEC) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(z + base + i);
+      const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+      for (int u = 0; u < N; ++u) to[u] = Elem<T>::load(e[u]);
+    } else {
+      to[0] = Elem<T>::load(z[base + i]);
+    }
+  };
   if constexpr (REGS > 0) {
 #pragma unroll
     for (int e = 0; e < REGS; ++e) {
-      const int i = threadIdx.x + e * 256;
-      held[e] = i < dim ? Elem<T>::load(z[base + i]) : 0.f;
-      take(held[e]);
+      const int i = (threadIdx.x + e * 256) * N;
+      if (i < dim) load(i, held + e * N);
+      else
+#pragma unroll
+        for (int u = 0; u < N; ++u) held[e * N + u] = 0.f;
+#pragma unroll
+      for (int u = 0; u < N; ++u) take(held[e * N + u]);
     }
   } else {
-    for (int i = threadIdx.x; i < dim; i += 256) take(Elem<T>::load(z[base + i]));
+    for (int i = threadIdx.x * N; i < dim; i += 256 * N) {
+      load(i, held);
+#pragma unroll
+      for (int u = 0; u < N; ++u) take(held[u]);
+    }
   }
   block_sum3_256(s2, s4, s6, part);
   const float n = (float)dim;
   const float r1 = coef[0] / sqrtf(s2 / n + eps), r2 = coef[1] / sqrtf(s4 / n + eps), r3 = coef[2] / sqrtf(s6 / n + eps);
   const float e0 = coef[3];
-  auto emit = [&](int i, float v) { y[base + i] = Elem<T>::store(((r1 * v + r2 * (v * v)) + r3 * (v * v * v)) + e0); };
+  auto emit = [&](int i, const float* v) {
+    if constexpr (VEC) {
+      uint4 out;
+      T* o = reinterpret_cast<T*>(&out);
+#pragma unroll
+      for (int u = 0; u < N; ++u) o[u] = Elem<T>::store(((r1 * v[u] + r2 * (v[u] * v[u])) + r3 * (v[u] * v[u] * v[u])) + e0);
+      *reinterpret_cast<uint4*>(y + base + i) = out;
+    } else {
+      y[base + i] = Elem<T>::store(((r1 * v[0] + r2 * (v[0] * v[0])) + r3 * (v[0] * v[0] * v[0])) + e0);
+    }
+  };
   if constexpr (REGS > 0) {
 #pragma unroll
     for (int e = 0; e < REGS; ++e) {
-      const int i = threadIdx.x + e * 256;
-      if (i < dim) emit(i, held[e]);
+      const int i = (threadIdx.x + e * 256) * N;
+      if (i < dim) emit(i, held + e * N);
     }
   } else {
-    for (int i = threadIdx.x; i < dim; i += 256) emit(i, Elem<T>::load(z[base + i]));
+    for (int i = threadIdx.x * N; i < dim; i += 256 * N) {
+      load(i, held);
+      emit(i, held);
+    }
   }
 }
 
 #define ROUTE_MAX_E 1024
 
-// One block of 64 threads a token. s = sigmoid(logit); choice = s + correction; groups of neighbours are ranked by the
-// sum of their two largest choices and the `keep` best stay open; the `top` largest open choices are chosen (equal
-// ones: the lower index first); weight = s * scale for a chosen expert, 0 for every other.
+// The router's choice for one token, by all threads of a block: score_s holds s = sigmoid(logit), choice_s the choice
+// scores s + correction. Groups of neighbours are ranked by the sum of their two largest choices and the `keep` best
+// stay open; the `top` largest open choices are chosen (equal ones: the lower index first); weight = s * scale for a
+// chosen expert, 0 for every other.
+__device__ __forceinline__ void route_token(float* score_s, float* choice_s, float* group_s, float* __restrict__ weights,
+                                            int experts, int top, int groups, int keep, float scale) {
+  const int step = blockDim.x;
+  if (groups > 1) {
+    const int size = experts / groups;
+    for (int g = threadIdx.x; g < groups; g += step) {
+      float a = -INFINITY, b = -INFINITY;                // the two largest of the group
+      for (int i = 0; i < size; ++i) {
+        const float v = choice_s[g * size + i];
+        if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+      }
+      group_s[g] = size > 1 ? a + b : a;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < experts; e += step) {
+      const int g = e / size;
+      const float mine = group_s[g];
+      int ahead = 0;
+      for (int o = 0; o < groups; ++o) ahead += (group_s[o] > mine) || (group_s[o] == mine && o < g);
+      if (ahead >= keep) choice_s[e] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  for (int e = threadIdx.x; e < experts; e += step) {
+    const float mine = choice_s[e];
+    int ahead = 0;
+    for (int o = 0; o < experts; ++o) ahead += (choice_s[o] > mine) || (choice_s[o] == mine && o < e);
+    weights[e] = (ahead < top && mine > -INFINITY) ? score_s[e] * scale : 0.f;
+  }
+}
+
+// One block of 64 threads a token, from logits.
 __global__ void __launch_bounds__(64) moe_route_kernel(const float* __restrict__ logits,
                                                        const float* __restrict__ correction, float* __restrict__ weights,
                                                        int experts, int top, int groups, int keep, float scale) {
@@ -72,50 +139,80 @@ __global__ void __launch_bounds__(64) moe_route_kernel(const float* __restrict__
     choice_s[e] = correction ? s + correction[e] : s;
   }
   __syncthreads();
-  if (groups > 1) {
-    const int size = experts / groups;
-    for (int g = threadIdx.x; g < groups; g += 64) {
-      float a = -INFINITY, b = -INFINITY;                // the two largest of the group
-      for (int i = 0; i < size; ++i) {
-        const float v = choice_s[g * size + i];
-        if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+  route_token(score_s, choice_s, group_s, weights + base, experts, top, groups, keep, scale);
+}
+
+// One block of 256 threads a token, from the token's row: the float32 logits x . router[e] first (the row waits in LDS
+// as float32; wave w takes experts w, w + 4, ..., its lanes a 64th of the row each, added up in an order the width
+// alone decides), then the choice.
+template <typename T>
+__global__ void __launch_bounds__(256) moe_router_kernel(const T* __restrict__ x, const float* __restrict__ router,
+                                                         const float* __restrict__ correction,
+                                                         float* __restrict__ weights, int width, int experts, int top,
+                                                         int groups, int keep, float scale) {
+  extern __shared__ float xs[];                          // [width]
+  __shared__ float score_s[ROUTE_MAX_E];
+  __shared__ float choice_s[ROUTE_MAX_E];
+  __shared__ float group_s[ROUTE_MAX_E];
+  const int64_t t = blockIdx.x;
+  for (int i = threadIdx.x; i < width; i += 256) xs[i] = Elem<T>::load(x[t * width + i]);
+  __syncthreads();
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const bool wide = width % 4 == 0 && (uintptr_t)router % 16 == 0;
+  for (int e = wave; e < experts; e += 4) {
+    const float* w = router + (int64_t)e * width;
+    float acc = 0.f;
+    if (wide) {
+      for (int i = lane * 4; i < width; i += WAVE * 4) {
+        const float4 v = *reinterpret_cast<const float4*>(w + i);
+        acc += xs[i] * v.x + xs[i + 1] * v.y + xs[i + 2] * v.z + xs[i + 3] * v.w;
       }
-      group_s[g] = size > 1 ? a + b : a;
+    } else {
+      for (int i = lane; i < width; i += WAVE) acc += xs[i] * w[i];
     }
-    __syncthreads();
-    for (int e = threadIdx.x; e < experts; e += 64) {
-      const int g = e / size;
-      const float mine = group_s[g];
-      int ahead = 0;
-      for (int o = 0; o < groups; ++o) ahead += (group_s[o] > mine) || (group_s[o] == mine && o < g);
-      if (ahead >= keep) choice_s[e] = -INFINITY;
+    acc = wave_sum(acc);
+    if (lane == 0) {
+      const float s = 1.0f / (1.0f + expf(-acc));
+      score_s[e] = s;
+      choice_s[e] = correction ? s + correction[e] : s;
     }
-    __syncthreads();
   }
-  for (int e = threadIdx.x; e < experts; e += 64) {
-    const float mine = choice_s[e];
-    int ahead = 0;
-    for (int o = 0; o < experts; ++o) ahead += (choice_s[o] > mine) || (choice_s[o] == mine && o < e);
-    weights[base + e] = (ahead < top && mine > -INFINITY) ? score_s[e] * scale : 0.f;
-  }
+  __syncthreads();
+  route_token(score_s, choice_s, group_s, weights + t * experts, experts, top, groups, keep, scale);
 }
 
 // y[t, c] = round(round(silu(gate)) * up) * weight of the column's expert, 0 where that weight is 0; columns from
-// experts * ff on belong to an expert every token uses with weight 1.
-template <typename T>
+// experts * ff on belong to an expert every token uses with weight 1. VEC: a thread takes 16 bytes of a row at a time
+// (every row and the border between gates and ups fall on 16 bytes, and a group of columns is one expert's).
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(256) moe_gate_kernel(const T* __restrict__ gate_up, const float* __restrict__ weights,
                                                        T* __restrict__ y, int experts, int ff, int shared) {
   const int cols = experts * ff + shared;
   const int64_t t = blockIdx.y;
   const T* row = gate_up + t * 2 * cols;
-  for (int c = blockIdx.x * 256 + threadIdx.x; c < cols; c += gridDim.x * 256) {
+  constexpr int N = VEC ? Elem<T>::kVec : 1;
+  for (int c = (blockIdx.x * 256 + threadIdx.x) * N; c < cols; c += gridDim.x * 256 * N) {
     const float w = c < experts * ff ? weights[t * experts + c / ff] : 1.0f;
-    float out = 0.f;
-    if (w != 0.f) {
-      const float g = Elem<T>::load(row[c]), u = Elem<T>::load(row[cols + c]);
-      out = Elem<T>::round(Elem<T>::round(silu<T>(g)) * u) * w;
+    if constexpr (VEC) {
+      uint4 out = make_uint4(0u, 0u, 0u, 0u);
+      if (w != 0.f) {
+        const uint4 graw = *reinterpret_cast<const uint4*>(row + c), uraw = *reinterpret_cast<const uint4*>(row + cols + c);
+        const T* g = reinterpret_cast<const T*>(&graw);
+        const T* u = reinterpret_cast<const T*>(&uraw);
+        T* o = reinterpret_cast<T*>(&out);
+#pragma unroll
+        for (int i = 0; i < N; ++i)
+          o[i] = Elem<T>::store(Elem<T>::round(Elem<T>::round(silu<T>(Elem<T>::load(g[i]))) * Elem<T>::load(u[i])) * w);
+      }
+      *reinterpret_cast<uint4*>(y + t * cols + c) = out;
+    } else {
+      float out = 0.f;
+      if (w != 0.f) {
+        const float g = Elem<T>::load(row[c]), u = Elem<T>::load(row[cols + c]);
+        out = Elem<T>::round(Elem<T>::round(silu<T>(g)) * u) * w;
+      }
+      y[t * cols + c] = Elem<T>::store(out);
     }
-    y[t * cols + c] = Elem<T>::store(out);
   }
 }
 }  // namespace
@@ -125,9 +222,22 @@ extern "C" int holon_polynorm(const void* z, const float* coef, void* y, int64_t
   HOLON_CHECK(rows >= 0 && rows <= 0x7fffffffLL && dim > 0, "polynorm: rows=%lld dim=%d", (long long)rows, dim);
   if (rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-#define PN(T, R) polynorm_kernel<T, R><<<(unsigned)rows, 256, 0, s>>>((const T*)z, coef, (T*)y, dim, eps)
-  if (dtype == HOLON_F32) { if (dim <= 1024) PN(float, 4); else if (dim <= 8192) PN(float, 32); else PN(float, 0); }
-  else { if (dim <= 1024) PN(bf16_t, 4); else if (dim <= 8192) PN(bf16_t, 32); else PN(bf16_t, 0); }
+  // in groups of 16 bytes where every row starts on such a border; the sums then run in another order than value by
+  // value, but still in one that the width alone decides
+  const int vec = dtype == HOLON_F32 ? 4 : 8;
+  const bool wide = dim % vec == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)y % 16 == 0;
+  const int groups = wide ? dim / vec : dim;
+#define PN(T, R, V) polynorm_kernel<T, R, V><<<(unsigned)rows, 256, 0, s>>>((const T*)z, coef, (T*)y, dim, eps)
+#define PN_BY_SIZE(T, V)                      \
+  do {                                        \
+    if (groups <= 256) PN(T, 1, V);           \
+    else if (groups <= 1024) PN(T, 4, V);     \
+    else if (!V && groups <= 4096) PN(T, 16, V); \
+    else PN(T, 0, V);                         \
+  } while (0)
+  if (dtype == HOLON_F32) { if (wide) PN_BY_SIZE(float, true); else PN_BY_SIZE(float, false); }
+  else { if (wide) PN_BY_SIZE(bf16_t, true); else PN_BY_SIZE(bf16_t, false); }
+#undef PN_BY_SIZE
 #undef PN
   HOLON_LAUNCH_OK();
   return 0;
@@ -146,6 +256,28 @@ extern "C" int holon_moe_route(const float* logits, const float* correction, flo
   return 0;
 }
 
+extern "C" int holon_moe_router(const void* x, const float* router, const float* correction, float* weights,
+                                int64_t rows, int width, int experts, int top, int groups, int keep, float scale,
+                                int dtype, void* stream) {
+  HOLON_CHECK(rows >= 0 && rows <= 0x7fffffffLL && width >= 1 && width <= 12288 && experts >= 1 &&
+                  experts <= ROUTE_MAX_E && top >= 1 && top <= experts,
+              "moe_router: rows=%lld of %d (at most 12,288), top %d of %d experts (at most %d)", (long long)rows, width,
+              top, experts, ROUTE_MAX_E);
+  HOLON_CHECK(groups <= 1 || (experts % groups == 0 && keep >= 1 && keep <= groups),
+              "moe_router: %d experts in %d groups of which %d stay open", experts, groups, keep);
+  if (rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t lds = (size_t)width * sizeof(float);
+  if (dtype == HOLON_F32)
+    moe_router_kernel<float><<<(unsigned)rows, 256, lds, s>>>((const float*)x, router, correction, weights, width,
+                                                             experts, top, groups, keep, scale);
+  else
+    moe_router_kernel<bf16_t><<<(unsigned)rows, 256, lds, s>>>((const bf16_t*)x, router, correction, weights, width,
+                                                              experts, top, groups, keep, scale);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
 extern "C" int holon_moe_gate(const void* gate_up, const float* weights, void* y, int64_t rows, int experts, int ff,
                               int shared, int dtype, void* stream) {
   HOLON_CHECK(rows >= 0 && rows <= 65535 * 1024LL && experts >= 1 && ff >= 1 && shared >= 0,
@@ -155,13 +287,16 @@ extern "C" int holon_moe_gate(const void* gate_up, const float* weights, void* y
   const int cols = experts * ff + shared;
   for (int64_t r0 = 0; r0 < rows; r0 += 65535) {
     const int n = (int)(rows - r0 < 65535 ? rows - r0 : 65535);
-    const dim3 grid((cols + 255) / 256 < 64 ? (cols + 255) / 256 : 64, n);
-    if (dtype == HOLON_F32)
-      moe_gate_kernel<float><<<grid, 256, 0, s>>>((const float*)gate_up + r0 * 2 * cols, weights + r0 * experts,
-                                                   (float*)y + r0 * cols, experts, ff, shared);
-    else
-      moe_gate_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)gate_up + r0 * 2 * cols, weights + r0 * experts,
-                                                    (bf16_t*)y + r0 * cols, experts, ff, shared);
+    const int vec = dtype == HOLON_F32 ? 4 : 8;
+    const bool wide = ff % vec == 0 && shared % vec == 0 && (uintptr_t)gate_up % 16 == 0 && (uintptr_t)y % 16 == 0;
+    const int groups = wide ? cols / vec : cols;
+    const dim3 grid((groups + 255) / 256 < 64 ? (groups + 255) / 256 : 64, n);
+#define MOE_GATE(T, V)                                                                                        \
+  moe_gate_kernel<T, V><<<grid, 256, 0, s>>>((const T*)gate_up + r0 * 2 * cols, weights + r0 * experts,       \
+                                             (T*)y + r0 * cols, experts, ff, shared)
+    if (dtype == HOLON_F32) { if (wide) MOE_GATE(float, true); else MOE_GATE(float, false); }
+    else { if (wide) MOE_GATE(bf16_t, true); else MOE_GATE(bf16_t, false); }
+#undef MOE_GATE
   }
   HOLON_LAUNCH_OK();
   return 0;

@@ -320,6 +320,10 @@ int holon_polynorm(const void* z, const float* coef, void* y, int64_t rows, int 
 // a chosen expert's weight is score * scale, every other 0.
 int holon_moe_route(const float* logits, const float* correction, float* weights, int64_t rows, int experts, int top,
                     int groups, int keep, float scale, void* stream);
+// The same from the tokens' rows x [rows, width] (float32 or bfloat16): the float32 logits x . router[e] (router
+// [experts, width] float32) and the choice, in one kernel.
+int holon_moe_router(const void* x, const float* router, const float* correction, float* weights, int64_t rows,
+                     int width, int experts, int top, int groups, int keep, float scale, int dtype, void* stream);
 // gate_up [rows, 2 C], C = experts ff + shared: y [rows, C] = silu(gate) up times the weight of the column's expert
 // (the last `shared` columns: 1), exactly 0 where the weight is 0.
 int holon_moe_gate(const void* gate_up, const float* weights, void* y, int64_t rows, int experts, int ff, int shared,

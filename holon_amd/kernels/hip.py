@@ -78,6 +78,10 @@ class HipKernels:
                                                   _P, _P],
             "holon_attention_decode_sink_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
                                                  _P, _P, _I, _I, _I, _I, _P, _P],
+            "holon_attention_prefill_mod_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I,
+                                                 _P, _F, _P, _P, _I, _P],
+            "holon_attention_decode_mod_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
+                                                _P, _P, _I, _I, _I, _I, _P, _F, _P, _P, _I, _P],
             "holon_attention_decode_fused_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
                                                   _P, _P, _F, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P],
             "holon_gemm_skinny_supported": [_I, _I, _I],
@@ -638,7 +642,8 @@ class HipKernels:
     def attention_on_cores(self, head_dim, page_size, dtype) -> bool:
         return bool(dtype in _DT and self.lib.holon_attention_mfma_supported(head_dim, page_size, _DT[dtype]))
 
-    def paged_attention(self, q, pages, table, rows: AttnRows, page_size, scale, window, sink=None):
+    def paged_attention(self, q, pages, table, rows: AttnRows, page_size, scale, window, sink=None, softcap=0.0,
+                        dist=None, keep_first=0):
         self._check(q, "attention q")
         self._check(pages, "attention pages", q.dtype)
         self._check(table, "block table", torch.int32)
@@ -652,6 +657,33 @@ class HipKernels:
             self._check(sink, "attention sink", torch.float32)
             if sink.shape != (hq,):
                 raise KernelError(f"attention: sink {tuple(sink.shape)} for {hq} heads")
+        changed = bool(softcap) or dist is not None or (window > 0 and keep_first > 0)
+        if dist is not None:
+            for v in dist:
+                self._check(v, "attention distance bias", torch.float32)
+                if v.shape != (hq,):
+                    raise KernelError(f"attention: a distance bias of {tuple(v.shape)} for {hq} heads")
+        if changed and not self.lib.holon_attention_mfma_supported(d, page_size, self._dt(q, "attention")):
+            raise KernelError("attention: a cap, a distance bias and kept first tokens are served by the matrix-core "
+                              f"kernels (and by `softmax_attention`), not at head_dim {d}, page {page_size}, {q.dtype}")
+        if changed:
+            common = (q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(), table.shape[1],
+                      rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr())
+            mod = (float(softcap), _ptr(dist[0]) if dist is not None else None,
+                   _ptr(dist[1]) if dist is not None else None, int(keep_first) if window > 0 else 0)
+            if rows.n_chunk:
+                self._call(self.lib.holon_attention_prefill_mod_bf16, *common, rows.chunk_rows.data_ptr(), rows.n_chunk,
+                           rows.max_chunk_query, rows.max_chunk_len, hq, hkv, d, page_size, float(scale), int(window),
+                           _ptr(sink), *mod, self._stream())
+            if rows.n_decode:
+                span = rows.max_decode_len if not window else min(rows.max_decode_len, window + 31)
+                splits, per, waves = self.decode_splits(rows.n_decode * hkv * ((hq // hkv + 15) // 16), span, d)
+                part_o, part_ml = self._decode_parts(rows.n_decode * hq * (splits // waves), d, q.device)
+                self._call(self.lib.holon_attention_decode_mod_bf16, *common, rows.decode_rows.data_ptr(),
+                           rows.n_decode, rows.max_decode_len, hq, hkv, d, page_size, float(scale), int(window),
+                           _ptr(part_o), _ptr(part_ml), splits, per, waves, int(rows.in_order and rows.n_decode == t),
+                           _ptr(sink), *mod, self._stream())
+            return out
         if self.lib.holon_attention_mfma_supported(d, page_size, self._dt(q, "attention")):
             common = (q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(), table.shape[1],
                       rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr())

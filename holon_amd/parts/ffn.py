@@ -118,6 +118,26 @@ def _moe_route_hip(launch, logits, correction, top, groups, keep, scale):
     return w
 
 
+def moe_router_plain(x, router, correction, top, groups, keep, scale):
+    """x [T, W] (any dtype), router [E, W] float32: the float32 logits x . router[e], then `moe_route` on them."""
+    return moe_route_plain(x.float() @ router.float().T, correction, top, groups, keep, scale)
+
+
+def _moe_router_hip(launch, x, router, correction, top, groups, keep, scale):
+    (t, w), e = x.shape, router.shape[0]
+    _need(x.is_cuda and x.is_contiguous() and x.dtype in _DT and router.is_contiguous() and router.dtype == torch.float32
+          and router.shape == (e, w) and 1 <= top <= e <= 1024 and w <= 12288
+          and (correction is None or (correction.dtype == torch.float32 and correction.is_contiguous()
+                                      and correction.shape == (e,)))
+          and (groups <= 1 or (e % groups == 0 and 1 <= keep <= groups)),
+          f"moe_router: rows {tuple(x.shape)} {x.dtype}, {e} experts, top {top}, {groups} groups of which {keep}")
+    weights = torch.empty((t, e), dtype=torch.float32, device=x.device)
+    if t:
+        launch(x.data_ptr(), router.data_ptr(), None if correction is None else correction.data_ptr(),
+               weights.data_ptr(), t, w, e, int(top), int(groups), int(keep), float(scale), _DT[x.dtype])
+    return weights
+
+
 def moe_gate_plain(gate_up, weights, ff, shared):
     """gate_up [T, 2 C] with C = E ff + shared columns of gates, then as many of ups; weights [T, E] float32.
     -> [T, C]: silu(gate) * up (as `silu_mul` rounds it), times the weight of the column's expert (column c belongs to
@@ -148,6 +168,8 @@ def _moe_gate_hip(launch, gate_up, weights, ff, shared):
 register_kernel(KernelOp("polynorm", polynorm_plain, "holon_polynorm", [_P, _P, _P, _L, _I, _F, _I], _polynorm_hip))
 register_kernel(KernelOp("moe_route", moe_route_plain, "holon_moe_route", [_P, _P, _P, _L, _I, _I, _I, _I, _F],
                          _moe_route_hip))
+register_kernel(KernelOp("moe_router", moe_router_plain, "holon_moe_router",
+                         [_P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _F, _I], _moe_router_hip))
 register_kernel(KernelOp("moe_gate", moe_gate_plain, "holon_moe_gate", [_P, _P, _P, _L, _I, _I, _I, _I], _moe_gate_hip))
 
 
@@ -175,7 +197,8 @@ class PolyNormFFN(Part):
 class MoE(Part):
     """A mixture of SiLU-gated experts with a sigmoid router, and an optional shared expert that every token uses.
 
-    Router: float32 logits, scores s = sigmoid(logits); experts are chosen by s + `correction` (`bias`), optionally
+    Router: float32 logits (products of the input as it is with float32 weights, summed in float32), scores s =
+    sigmoid(logits); experts are chosen by s + `correction` (`bias`), optionally
     only within the `keep` best of `groups` groups of neighbouring experts, `top` per token; a chosen expert's output
     is weighted by s * `scale`. All experts' gate and up projections are one product and all down projections
     another: the activations of experts a token did not choose are set to 0 in between (`moe_gate`), so the second
@@ -232,9 +255,8 @@ class MoE(Part):
 
     def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
         k = self.kernels
-        logits = k.linear(x if x.dtype == torch.float32 else k.widen_rows(x), self.router)
-        weights = k.moe_route(logits, self.correction if self.has_bias else None, self.top, self.groups, self.keep,
-                              self.scale)
+        weights = k.moe_router(x, self.router, self.correction if self.has_bias else None, self.top, self.groups,
+                               self.keep, self.scale)
         act = k.moe_gate(self.gate_up(x), weights, self.inter, self.shared)
         return self.all_down(act)
 

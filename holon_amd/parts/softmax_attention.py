@@ -268,13 +268,13 @@ register_kernel(KernelOp("latent_prepare", latent_prepare_plain, "holon_latent_p
 
 def attend(k, q, held, view, step, kv_heads, vdim, sink, scale, window, softcap=0.0, dist=None, keep_first=0):
     """The attention of both mixers: on the matrix cores where keys and values have one width that those kernels
-    serve (the pages' layout is then theirs) and the scores are plain scaled products under a plain window, else the
-    general kernel. q [T, H, D] -> [T, H V]."""
+    serve (the pages' layout is then theirs), else the general kernel. q [T, H, D] -> [T, H V]."""
     t, heads, dim = q.shape
-    plain = not softcap and dist is None and not (window > 0 and keep_first > 0)
-    if plain and dim == vdim and k.attention_on_cores(dim, view.page_size, q.dtype):
+    if dim == vdim and k.attention_on_cores(dim, view.page_size, q.dtype):
         pages = held.pages.view(-1, 2, kv_heads, view.page_size * dim)
-        return k.paged_attention(q, pages, view.table, step.rows, view.page_size, scale, window, sink=sink).view(t, heads * vdim)
+        return k.paged_attention(q, pages, view.table, step.rows, view.page_size, scale, window, sink=sink,
+                                 softcap=softcap, dist=dist, keep_first=keep_first if window > 0 else 0
+                                 ).view(t, heads * vdim)
     return k.softmax_attention(q, held.pages, view.table, step.rows, step.token_row, step.positions, kv_heads, vdim,
                                view.page_size, sink, scale, window, softcap=softcap, dist=dist,
                                keep_first=keep_first if window > 0 else 0)

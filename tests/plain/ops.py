@@ -170,7 +170,8 @@ class TorchKernels:
     def attention_on_cores(self, head_dim, page_size, dtype):
         return self.cores
 
-    def paged_attention(self, q, pages, table, rows, page_size, scale, window, sink=None):
+    def paged_attention(self, q, pages, table, rows, page_size, scale, window, sink=None, softcap=0.0, dist=None,
+                        keep_first=0):
         t, hq, d = q.shape
         hkv = pages.shape[2]
         kp = pages[:, 0].view(-1, hkv, page_size, d)
@@ -187,9 +188,14 @@ class TorchKernels:
             scores = torch.einsum("qhd,khd->hqk", _up(q[s:e]), k) * scale
             pos = torch.arange(n - (e - s), n, device=q.device)[:, None]
             key = torch.arange(n, device=q.device)[None, :]
+            if softcap:
+                scores = softcap * torch.tanh(scores / softcap)
+            if dist is not None:
+                far = (pos - key).clamp(min=0).to(scores.dtype)
+                scores = scores - _up(dist[0])[:, None, None] * torch.log1p(_up(dist[1])[:, None, None] * far)
             hidden = key > pos
             if window:
-                hidden = hidden | (pos - key >= window)
+                hidden = hidden | ((pos - key >= window) & (key >= keep_first))
             scores = scores.masked_fill(hidden, float("-inf"))
             if sink is not None:             # a column of its own in the softmax, dropped again: it has no value
                 scores = torch.cat((scores, _up(sink)[:, None, None].expand(hq, e - s, 1)), dim=-1)

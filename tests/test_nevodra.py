@@ -135,6 +135,66 @@ def test_float32_does_not_depend_on_the_cut(folders, device):
             assert H.rel_rms(row, whole[key]) < 1e-5, f"{key}: logits depend on how the prompt was cut"
 
 
+def test_the_matrix_core_path_of_the_mixers_on_the_twin(folders):
+    """Where keys and values have one width that the matrix-core attention kernels serve, both mixers hand their pages
+    to `paged_attention` (the cap, the distance bias and the kept tokens; the sink); the twin is told to say it serves
+    them, and the logits stay the plain model's."""
+    folder, requests = folders["D-sharp"], _requests("D-sharp", (70, 33, 58))
+    from holon_amd.engine.loading import load_model
+    from holon_amd.engine.replay import Replayer
+    kernels = TorchKernels()
+    kernels.cores = True
+    rep = Replayer(load_model(folder, device="cpu", dtype="float32", kernels=kernels, page_size=16, max_seqs=3,
+                              max_model_len=128, max_step_tokens=128, cache_tokens=192))
+    got = H.run_trace(rep, H.trace_mixed(requests, seed=2, max_live=3, decode_tail=5))
+    _check(folder, "float32", requests, got, "matrix-core path on the twin")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dim", [64, 128, 256])
+def test_changed_scores_on_the_matrix_cores(dim):
+    """`paged_attention` with a cap, a distance bias, kept first tokens and a sink, in bfloat16 at every head size the
+    matrix cores serve, prompt portions beside decode rows over scattered pages, against the plain form in float64."""
+    from holon_amd.kernels import load_hip
+    from holon_amd.kernels.api import AttnRows
+    k, dev, page, heads, groups = load_hip(), "cuda", 16, 4, 2
+    g = torch.Generator().manual_seed(dim)
+    lens, counts = [300, 75, 190, 33, 129], [300, 1, 60, 1, 1]          # tokens a row holds, and brings in this step
+    n_pages = sum(-(-n // page) for n in lens) + 1
+    table = torch.full((len(lens) + 1, 24), n_pages - 1, dtype=torch.int32)
+    order, at = torch.randperm(n_pages - 1, generator=g).tolist(), 0
+    for s_, n in enumerate(lens):
+        for i in range(-(-n // page)):
+            table[s_, i] = order[at]
+            at += 1
+    pages = (torch.randn(n_pages, 2, groups, page * dim, generator=g) * 0.5).to(dev).bfloat16()
+    qstart = [0]
+    for c in counts:
+        qstart.append(qstart[-1] + c)
+    q = torch.randn(qstart[-1], heads, dim, generator=g).to(dev).bfloat16()
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)          # noqa: E731
+    decode = [b for b, c in enumerate(counts) if c == 1]
+    chunk = [b for b, c in enumerate(counts) if c > 1]
+    rows = AttnRows(slots=i32(list(range(len(lens)))), lens=i32(lens), query_start=i32(qstart), decode_rows=i32(decode),
+                    chunk_rows=i32(chunk), n_decode=len(decode), n_chunk=len(chunk),
+                    max_decode_len=max(lens[b] for b in decode), max_chunk_query=max(counts),
+                    max_chunk_len=max(lens[b] for b in chunk))
+    r1, r2 = torch.rand(heads, generator=g).to(dev), (2 * torch.rand(heads, generator=g)).to(dev)
+    sink = torch.randn(heads, generator=g).to(dev)
+    twin = TorchKernels()
+    scale = 2.0 * dim ** -0.5
+    for window, keep, cap, dist, sk in ((0, 0, 3.0, (r1, r2), None), (40, 5, 3.0, (r1, r2), sink), (100, 64, 0.0, None, None),
+                                        (33, 70, 2.0, (r1, r2), None), (64, 1, 0.0, (r1, r2), None), (17, 32, 5.0, None, sink)):
+        got = k.paged_attention(q, pages, table.to(dev), rows, page, scale, window, sink=sk, softcap=cap, dist=dist,
+                                keep_first=keep)
+        want = twin.paged_attention(q.double(), pages.double(), table.to(dev), rows, page, scale, window,
+                                    sink=None if sk is None else sk.double(), softcap=cap,
+                                    dist=None if dist is None else (dist[0].double(), dist[1].double()), keep_first=keep)
+        assert H.rel_rms(got, want) < 8e-3, (dim, window, keep, cap)
+        per = ((got.double() - want).square().mean((1, 2)).sqrt() / want.square().mean().sqrt()).max().item()
+        assert per < 4e-2, (dim, window, keep, cap, per)
+
+
 @pytest.mark.parametrize("device", DEVICES)
 def test_the_stream_after_every_layer_run(folders, device):
     """The residual stream after each run of a layer (a repeated layer counts each time), float32, against the plain
@@ -160,18 +220,19 @@ def test_the_stream_after_every_layer_run(folders, device):
         assert H.rel_rms(x.cpu(), ref) < 2e-5, f"run {site.run} (layer {site.layer}, pass {site.turn})"
 
 
-def _needle_attention(root, size, keep_first, page):
+def _needle_attention(root, size, keep_first, page, dim=16, vdim=8):
     """One attention layer without filter, cap and distance bias (a score depends on the two tokens alone). A pair of
     token ids (query token, key token) whose score is the largest of all, and a filler token whose scores with them
     and with itself are lowest, with the queries' norm weight scaled until the pair's weight among a window of fillers
-    is nearly all of it. Returns the folder and the three ids."""
-    cfg = M.model(32, 40, [M.attention(2, 1, 16, 8, 0.25, size=size, keep_first=keep_first)], taps=0)
+    is nearly all of it. Returns the folder and the three ids. (Heads of 64 with keys and values of one width take the
+    matrix-core kernels in bfloat16 on the GPU.)"""
+    cfg = M.model(32, 40, [M.attention(2, 1, dim, vdim, 0.25, size=size, keep_first=keep_first)], taps=0)
     found = {}
 
     def edit(t):
         p = {k: v.double() for k, v in t.items()}
         a_in = plain.rms(p["embed"] * 2.0, 1e-6) * p["l0.norm1"]           # every token's mixer input
-        q = (plain.rms(a_in @ p["l0.mix.q"].T, 1e-6) * p["l0.mix.q.norm"]).view(-1, 2, 16)
+        q = (plain.rms(a_in @ p["l0.mix.q"].T, 1e-6) * p["l0.mix.q.norm"]).view(-1, 2, dim)
         k = plain.rms(a_in @ p["l0.mix.k"].T, 1e-6) * p["l0.mix.k.norm"]
         score = torch.einsum("ahd,bd->abh", q, k)[..., 0] * 0.25            # head 0: [query token, key token]
         a, b = divmod(int(score.argmax()), score.shape[1])
@@ -206,11 +267,11 @@ def _both_ways(folder, plain_model, device, dtype, page, cases, what):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("size,page", [(21, 8), (16, 16), (35, 16), (70, 32)])
-def test_a_key_just_inside_and_just_outside_the_window(tmp_path, size, page, dtype, device):
+@pytest.mark.parametrize("size,page,dim", [(21, 8, 16), (16, 16, 16), (35, 16, 16), (70, 32, 16), (35, 16, 64), (64, 16, 64)])
+def test_a_key_just_inside_and_just_outside_the_window(tmp_path, size, page, dim, dtype, device):
     """One key whose score stands out, `size - 1` and `size` tokens behind the query, on either side of a page border,
     behind a kept first token that is a filler."""
-    folder, a, b, filler = _needle_attention(tmp_path / "needle", size, 1, page)
+    folder, a, b, filler = _needle_attention(tmp_path / "needle", size, 1, page, dim, 8 if dim == 16 else dim)
     plain_model = M.PlainNevodra(folder)
     for key_at in (page - 1, page, 2 * page + 3):
         inside = [filler] * key_at + [b] + [filler] * (size - 2) + [a, filler]
@@ -221,11 +282,12 @@ def test_a_key_just_inside_and_just_outside_the_window(tmp_path, size, page, dty
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("keep,page", [(1, 8), (5, 8), (8, 8), (17, 16), (70, 16)])
-def test_the_last_kept_token_and_the_first_that_is_not(tmp_path, keep, page, dtype, device):
+@pytest.mark.parametrize("keep,page,dim", [(1, 8, 16), (5, 8, 16), (8, 8, 16), (17, 16, 16), (70, 16, 16), (4, 16, 64),
+                                           (32, 16, 64), (33, 16, 64), (70, 16, 64)])
+def test_the_last_kept_token_and_the_first_that_is_not(tmp_path, keep, page, dim, dtype, device):
     """A window of 10 that keeps the first `keep` tokens: the key whose score stands out as the last kept token and as
     the one after it, with the query 100 and more tokens later, many windows and freed pages away."""
-    folder, a, b, filler = _needle_attention(tmp_path / "kept", 10, keep, page)
+    folder, a, b, filler = _needle_attention(tmp_path / "kept", 10, keep, page, dim, 8 if dim == 16 else dim)
     plain_model = M.PlainNevodra(folder)
     n = keep + 100
     kept = [filler] * (keep - 1) + [b] + [filler] * (n - keep) + [a, filler]
@@ -504,6 +566,13 @@ def test_kernels_alone_against_their_plain_forms(dtype):
     gate_up = randn(9, 2 * (experts * ff + shared))
     weights = kernel_op("moe_route").plain(randn(9, experts, to=torch.float32), None, 2, 1, 1, 1.5)
     assert H.rel_rms(k.moe_gate(gate_up, weights, ff, shared), kernel_op("moe_gate").plain(gate_up, weights, ff, shared)) < tol
+    for experts, top, count, keep, width in ((8, 3, 2, 1, 256), (12, 4, 3, 2, 250), (64, 6, 8, 3, 2048), (5, 1, 1, 1, 77)):
+        x, router = randn(19, width), randn(experts, width, to=torch.float32) * 0.2
+        correction = randn(experts, to=torch.float32) * 0.5 - 0.4
+        got = k.moe_router(x, router, correction, top, count, keep, 1.7)
+        want = kernel_op("moe_router").plain(x, router, correction, top, count, keep, 1.7)
+        close = ((got != 0) != (want != 0)).any(1)            # rows whose choice fell the other way on a close call
+        assert close.sum() <= 1 and torch.allclose(got[~close], want[~close], atol=2e-5), (experts, width)
     x = randn(5, 77)
     assert torch.equal(k.scale_rows(x, 3.0), x.float() * 3.0)
     # a paged cache of three rows over scattered pages
