@@ -309,6 +309,13 @@ int holon_head_linear_rows(const void* x, const void* w, void* y, int rows, int 
 int holon_stream_rms(float* x32, const void* d1, int dt1, const void* d2, int dt2, const float* row, const void* w1,
                      const void* w2, int dtw, void* y1, void* y2, int64_t rows, int dim, float eps, int dt_out,
                      void* stream);
+// The same for a step of single tokens (row b is token b) whose results each go through a causal filter, y <- y +
+// conv(y), with the requests' last taps - 1 inputs in their slots (see parallel_block.hip).
+int holon_stream_rms_filter_supported(int dim, int taps);
+int holon_stream_rms_filter(float* x32, const void* d1, int dt1, const void* d2, int dt2, const float* row,
+                            const void* w1, const void* w2, int dtw, void* y1, void* y2, int64_t rows, int dim,
+                            float eps, int dt_out, const void* cw1, const void* cw2, void* held1, void* held2,
+                            const int32_t* slots, const int32_t* starts, int taps, void* stream);
 // y[i] = scale * x[i] as float32 (x float32 or bfloat16): a new copy.
 int holon_scale_rows(const void* x, float* y, int64_t n, int dtype, float scale, void* stream);
 

@@ -45,6 +45,52 @@ __global__ void causal_conv_kernel(const T* __restrict__ x, const T* __restrict_
   }
 }
 
+// The same for prompt portions with a thread taking 16 bytes of channels at a time (channels a multiple of that; rows
+// of x, y and the slots then start on 16-byte borders): the same products in the same order.
+template <typename T>
+__global__ void __launch_bounds__(256) causal_conv_wide_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                               const T* __restrict__ state, T* __restrict__ y,
+                                                               const int32_t* __restrict__ slots,
+                                                               const int32_t* __restrict__ starts,
+                                                               const int32_t* __restrict__ query_start,
+                                                               const int32_t* __restrict__ token_row, int channels,
+                                                               int taps, int add_input, int act) {
+  constexpr int N = Elem<T>::kVec;
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * N;
+  const int t = blockIdx.y;
+  if (c >= channels) return;
+  const int b = token_row[t];
+  const int q0 = query_start[b];
+  const int i = t - q0;
+  const bool carried = starts[b] > 0;
+  const T* held = state + (int64_t)slots[b] * (taps - 1) * channels;
+  float acc[N];
+#pragma unroll
+  for (int u = 0; u < N; ++u) acc[u] = 0.f;
+  uint4 last = make_uint4(0u, 0u, 0u, 0u);
+  for (int j = 0; j < taps; ++j) {
+    const int l = i - (taps - 1) + j;
+    uint4 raw = make_uint4(0u, 0u, 0u, 0u);
+    if (l >= 0) raw = *reinterpret_cast<const uint4*>(x + (int64_t)(q0 + l) * channels + c);
+    else if (carried) raw = *reinterpret_cast<const uint4*>(held + (int64_t)(taps - 1 + l) * channels + c);
+    const T* v = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+    for (int u = 0; u < N; ++u) acc[u] += Elem<T>::load(w[(int64_t)(c + u) * taps + j]) * Elem<T>::load(v[u]);
+    last = raw;
+  }
+  const T* own = reinterpret_cast<const T*>(&last);      // the last tap's input is the token itself
+  uint4 out;
+  T* o = reinterpret_cast<T*>(&out);
+#pragma unroll
+  for (int u = 0; u < N; ++u) {
+    float a = acc[u];
+    if (add_input) a += Elem<T>::load(own[u]);
+    if (act) a = silu<T>(a);
+    o[u] = Elem<T>::store(a);
+  }
+  *reinterpret_cast<uint4*>(y + (int64_t)t * channels + c) = out;
+}
+
 // After the filter has read the old inputs: the slot takes the row's last taps - 1 inputs, oldest first. A thread
 // moves its channel's entries in ascending order and reads only entries at or behind the one it writes.
 template <typename T>
@@ -593,9 +639,18 @@ extern "C" int holon_causal_conv(const void* x, const void* w, void* state, void
   const dim3 block(256), grid_t((channels + 255) / 256, tokens), grid_b((channels + 255) / 256, rows);
   HOLON_CHECK(!rows_in_order || tokens == rows, "causal_conv: rows in order means one token a row, got %d in %d", tokens,
               rows);
-  BY_DTYPE(dtype, (causal_conv_kernel<T><<<grid_t, block, 0, s>>>((const T*)x, (const T*)w, (T*)state, (T*)y, slots, starts,
-                                                                  query_start, token_row, channels, taps, add_input,
-                                                                  act, rows_in_order)));
+  const int vec = dtype == HOLON_F32 ? 4 : 8;
+  if (!rows_in_order && channels % vec == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0 &&
+      (uintptr_t)state % 16 == 0) {
+    const dim3 grid_w((channels / vec + 255) / 256, tokens);
+    BY_DTYPE(dtype, (causal_conv_wide_kernel<T><<<grid_w, block, 0, s>>>((const T*)x, (const T*)w, (const T*)state, (T*)y,
+                                                                         slots, starts, query_start, token_row,
+                                                                         channels, taps, add_input, act)));
+  } else {
+    BY_DTYPE(dtype, (causal_conv_kernel<T><<<grid_t, block, 0, s>>>((const T*)x, (const T*)w, (T*)state, (T*)y, slots,
+                                                                    starts, query_start, token_row, channels, taps,
+                                                                    add_input, act, rows_in_order)));
+  }
   HOLON_LAUNCH_OK();
   if (taps > 1 && !rows_in_order) {
     BY_DTYPE(dtype, (causal_conv_keep_kernel<T><<<grid_b, block, 0, s>>>((const T*)x, (T*)state, slots, starts,

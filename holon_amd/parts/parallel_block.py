@@ -82,6 +82,53 @@ def _stream_rms_hip(launch, x32, terms, row, w1, w2, eps, out_dtype):
     return y1, y2
 
 
+def stream_rms_filter_plain(x32, terms, row, w1, w2, eps, out_dtype, taps1, taps2, held1, held2, slots, starts):
+    """`stream_rms` for a step whose rows are single tokens (row b is token b), with each result y going through its
+    causal filter, y <- y + conv(y): `taps1`, `taps2` [W, taps] and the requests' last taps - 1 inputs `held1`, `held2`
+    [S, taps - 1, W] (ignored by a row that starts at 0; replaced afterwards), in `out_dtype`. The roundings are those
+    of the norm and the filter one after the other."""
+    from .convs import causal_conv_plain
+    a, b = stream_rms_plain(x32, terms, row, w1, w2, eps, out_dtype)
+    n = x32.shape[0]
+    order = torch.arange(n + 1, dtype=torch.int32, device=x32.device)
+    a = causal_conv_plain(a, taps1, held1, slots, starts, order, order[:n], n, True, False, True)
+    if b is not None:
+        b = causal_conv_plain(b, taps2, held2, slots, starts, order, order[:n], n, True, False, True)
+    return a, b
+
+
+def _stream_rms_filter_hip(launch, x32, terms, row, w1, w2, eps, out_dtype, taps1, taps2, held1, held2, slots, starts):
+    _need(x32.is_cuda and x32.is_contiguous() and x32.dtype == torch.float32 and x32.dim() == 2,
+          "stream_rms_filter: the stream is contiguous float32 rows on the GPU")
+    _need(len(terms) <= 2 and all(float(s) == 1.0 for _, s in terms), "stream_rms_filter: at most two terms, unscaled")
+    rows, dim = x32.shape
+    taps = taps1.shape[1]
+    ptrs, dts = [None, None], [0, 0]
+    for i, (term, _) in enumerate(terms):
+        _need(term.is_cuda and term.is_contiguous() and term.shape == x32.shape and term.dtype in _DT,
+              f"stream_rms_filter: term {i} must be contiguous rows of the stream's shape")
+        ptrs[i], dts[i] = term.data_ptr(), _DT[term.dtype]
+    _need(row is None or (row.is_cuda and row.is_contiguous() and row.dtype == torch.float32 and row.shape == (dim,)),
+          "stream_rms_filter: the added row is float32 of the stream's width")
+    _need(out_dtype in _DT and w1 is not None and w1.is_contiguous() and w1.shape == (dim,) and w1.dtype in _DT
+          and (w2 is None or (w2.is_contiguous() and w2.shape == (dim,) and w2.dtype == w1.dtype)),
+          "stream_rms_filter: weights of the rows' width")
+    for cw, held, there in ((taps1, held1, True), (taps2, held2, w2 is not None)):
+        _need(not there or (cw.is_contiguous() and cw.dtype == out_dtype and cw.shape == (dim, taps)
+                            and held.is_contiguous() and held.dtype == out_dtype
+                            and tuple(held.shape[1:]) == (taps - 1, dim)),
+              "stream_rms_filter: taps [W, taps] and held inputs [S, taps - 1, W] in the results' dtype")
+    _need(slots.dtype == torch.int32 and starts.dtype == torch.int32 and slots.shape[0] >= rows and starts.shape[0] >= rows,
+          "stream_rms_filter: a slot and a start for every row")
+    y1 = torch.empty((rows, dim), dtype=out_dtype, device=x32.device)
+    y2 = torch.empty((rows, dim), dtype=out_dtype, device=x32.device) if w2 is not None else None
+    if rows:
+        launch(x32.data_ptr(), ptrs[0], dts[0], ptrs[1], dts[1], _ptr(row), _ptr(w1), _ptr(w2), _DT[w1.dtype], _ptr(y1),
+               _ptr(y2), rows, dim, float(eps), _DT[out_dtype], taps1.data_ptr(), _ptr(taps2) if w2 is not None else None,
+               held1.data_ptr(), _ptr(held2) if w2 is not None else None, slots.data_ptr(), starts.data_ptr(), taps)
+    return y1, y2
+
+
 def scale_rows_plain(x, scale):
     """x [T, W] -> a new float32 tensor of scale * x."""
     return x.float() * scale
@@ -96,6 +143,9 @@ def _scale_rows_hip(launch, x, scale):
 
 register_kernel(KernelOp("stream_rms", stream_rms_plain, "holon_stream_rms",
                          [_P, _P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _L, _I, _F, _I], _stream_rms_hip))
+register_kernel(KernelOp("stream_rms_filter", stream_rms_filter_plain, "holon_stream_rms_filter",
+                         [_P, _P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _L, _I, _F, _I, _P, _P, _P, _P, _P, _P, _I],
+                         _stream_rms_filter_hip))
 register_kernel(KernelOp("scale_rows", scale_rows_plain, "holon_scale_rows", [_P, _P, _L, _I, _F], _scale_rows_hip))
 
 
@@ -153,12 +203,16 @@ class Parallel32(Part):
         if self.passes > 0:
             self.declare("step", (self.passes, hidden), kind=FLOAT32, init="zero")
         self._one_kernel: float | None = None      # the norms' eps when one kernel serves both
+        self._fused_filter = False                 # whether a step of single tokens runs norms and filters as one kernel
 
     def finalize(self) -> None:
         specs = [n.fusion() for n in (self.norm1, self.norm2) if n is not None]
         if all(sp is not None and sp.get("norm") == "rmsnorm" and sp["weight"] is not None for sp in specs) \
                 and len({sp["eps"] for sp in specs}) == 1:
             self._one_kernel = float(specs[0]["eps"])
+            # (the kernel serves widths that are a multiple of 4 up to 8,192 and up to four taps; the plain form any)
+            self._fused_filter = self.conv1 is not None and (self.ffn is None or self.conv2 is not None) \
+                and self.hidden % 4 == 0 and self.hidden <= 8192 and self.conv1.taps <= 4
 
     def state(self):
         return [s for conv in (self.conv1, self.conv2) if conv is not None for s in conv.state()] + \
@@ -176,6 +230,14 @@ class Parallel32(Part):
             row = self.step[site.turn]
         terms = _terms(stream.delta)
         stream.delta = stream.stats = None
+        if self._fused_filter and step.rows.in_order:      # single tokens: the norms and both filters in one kernel
+            second = self.conv2 is not None
+            a, b = k.stream_rms_filter(h, terms, row, self.norm1.weight, self.norm2.weight if second else None,
+                                       self._one_kernel, self.build.dtype, self.conv1.weight,
+                                       self.conv2.weight if second else None, site.slot_state[self.conv1.name],
+                                       site.slot_state[self.conv2.name] if second else None, step.slots, step.starts)
+            stream.delta = Pending([(t, 1.0) for t in self._mix(a, b, step, site)])
+            return stream
         if self._one_kernel is not None:
             a, b = k.stream_rms(h, terms, row, self.norm1.weight, self.norm2.weight if self.norm2 is not None else None,
                                 self._one_kernel, self.build.dtype)
@@ -186,12 +248,16 @@ class Parallel32(Part):
             b = self.norm2(h) if self.norm2 is not None else None
         if self.conv1 is not None:
             a = self.conv1(a, step, site)
-        out = [(self.mixer(a, step, site), 1.0)]
-        if self.ffn is not None:
-            if self.conv2 is not None:
-                b = self.conv2(b, step, site)
-            out.append((self.ffn(b, step), 1.0))
-        stream.delta = Pending(out)
+        if self.ffn is not None and self.conv2 is not None:
+            b = self.conv2(b, step, site)
+        stream.delta = Pending([(t, 1.0) for t in self._mix(a, b, step, site)])
         return stream
+
+    def _mix(self, a, b, step, site) -> list[torch.Tensor]:
+        """Both sublayers' results from their inputs."""
+        out = [self.mixer(a, step, site)]
+        if self.ffn is not None:
+            out.append(self.ffn(b, step))
+        return out
 
     __call__ = forward

@@ -559,6 +559,21 @@ def test_kernels_alone_against_their_plain_forms(dtype):
         a = k.stream_rms(xa, [(t1, 1.0), (t2, 1.0)], row, w1, w2, 1e-6, dtype)
         b = kernel_op("stream_rms").plain(xb, [(t1, 1.0), (t2, 1.0)], row, w1, w2, 1e-6, dtype)
         assert H.rel_rms(xa, xb) < 1e-6 and H.rel_rms(a[0], b[0]) < tol and H.rel_rms(a[1], b[1]) < tol, dim
+    for dim, taps in ((96, 3), (2048, 4), (252, 2), (5000, 1), (8192, 2)):      # single tokens: norms and filters in one kernel
+        if dim % 4:
+            continue
+        x, t1, t2 = randn(6, dim, to=torch.float32), randn(6, dim), randn(6, dim)
+        row, w1, w2 = randn(dim, to=torch.float32), randn(dim), randn(dim)
+        c1, c2 = randn(dim, taps) * 0.3, randn(dim, taps) * 0.3
+        held = [randn(9, taps - 1, dim) for _ in range(2)]
+        slots = torch.tensor([4, 0, 7, 2, 8, 1], dtype=torch.int32, device=dev)
+        starts = torch.tensor([3, 0, 1, 0, 9, 2], dtype=torch.int32, device=dev)
+        xa, xb, ha, hb = x.clone(), x.clone(), [h.clone() for h in held], [h.clone() for h in held]
+        a = k.stream_rms_filter(xa, [(t1, 1.0), (t2, 1.0)], row, w1, w2, 1e-6, dtype, c1, c2, ha[0], ha[1], slots, starts)
+        b = kernel_op("stream_rms_filter").plain(xb, [(t1, 1.0), (t2, 1.0)], row, w1, w2, 1e-6, dtype, c1, c2, hb[0], hb[1],
+                                                 slots, starts)
+        assert H.rel_rms(xa, xb) < 1e-6 and H.rel_rms(a[0], b[0]) < tol and H.rel_rms(a[1], b[1]) < tol, (dim, taps)
+        assert taps == 1 or (H.rel_rms(ha[0], hb[0]) < tol and H.rel_rms(ha[1], hb[1]) < tol), (dim, taps)
     for dim in (80, 321, 3000, 9000):
         z, coef = randn(5, dim), torch.tensor([0.5, -0.3, 0.2, 0.1], device=dev)
         assert H.rel_rms(k.polynorm(z, coef, 1e-6), kernel_op("polynorm").plain(z, coef, 1e-6)) < tol, dim
