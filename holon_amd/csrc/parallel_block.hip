@@ -117,22 +117,25 @@ struct Filters {
 template <int TAPS>
 struct Filter4 {
   float old[TAPS > 1 ? TAPS - 1 : 1][4];
+  float taps[TAPS][4];                                   // the four channels' taps as they lie: [channel][tap] flat
   int64_t base;
-  __device__ __forceinline__ void load(const void* held, int slot, bool carried, int c0, int dim, int dt) {
+  __device__ __forceinline__ void load(const void* held, const void* w, int slot, bool carried, int c0, int dim, int dt) {
     base = (int64_t)slot * (TAPS - 1) * dim + c0;
 #pragma unroll
     for (int j = 0; j + 1 < TAPS; ++j) {
       if (carried) load4(held, base + (int64_t)j * dim, dt, old[j]);
       else old[j][0] = old[j][1] = old[j][2] = old[j][3] = 0.f;
     }
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) load4(w, (int64_t)c0 * TAPS + 4 * j, dt, taps[j]);
   }
-  __device__ __forceinline__ void apply(const float (&a)[4], const void* w, int c0, int dt, float (&y)[4]) const {
+  __device__ __forceinline__ void apply(const float (&a)[4], float (&y)[4]) const {
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       float acc = 0.f;
 #pragma unroll
-      for (int j = 0; j + 1 < TAPS; ++j) acc += load_as(w, (int64_t)(c0 + u) * TAPS + j, dt) * old[j][u];
-      acc += load_as(w, (int64_t)(c0 + u) * TAPS + TAPS - 1, dt) * a[u];
+      for (int j = 0; j + 1 < TAPS; ++j) acc += taps[(u * TAPS + j) / 4][(u * TAPS + j) % 4] * old[j][u];
+      acc += taps[(u * TAPS + TAPS - 1) / 4][(u * TAPS + TAPS - 1) % 4] * a[u];
       y[u] = acc + a[u];
     }
   }
@@ -188,11 +191,22 @@ __global__ void __launch_bounds__(256) stream_rms_vec_kernel(float* __restrict__
     for (int u = 0; u < 4; ++u) sq += v[u] * v[u];
   }
   if (!w1) return;
+  constexpr bool FILTER = TAPS > 0;
+  // the filters' old inputs and taps are asked for now, so that they arrive while the row's sum is taken
+  Filter4<FILTER ? TAPS : 1> f1[FILTER ? REGS : 1], f2[FILTER ? REGS : 1];
+  if constexpr (FILTER) {
+    const int slot = f.slots[blockIdx.x];
+    const bool carried = f.starts[blockIdx.x] > 0;
+#pragma unroll
+    for (int e = 0; e < REGS; ++e) {
+      const int i = (threadIdx.x + e * 256) * 4;
+      if (i >= dim) continue;
+      f1[e].load(f.held1, f.w1, slot, carried, i, dim, dt_out);
+      if (w2) f2[e].load(f.held2, f.w2, slot, carried, i, dim, dt_out);
+    }
+  }
   sq = block_sum_256(sq, part);
   const float r = 1.0f / sqrtf(sq / (float)dim + eps);
-  constexpr bool FILTER = TAPS > 0;
-  const int slot = FILTER ? f.slots[blockIdx.x] : 0;
-  const bool carried = FILTER ? f.starts[blockIdx.x] > 0 : false;
 #pragma unroll
   for (int e = 0; e < REGS; ++e) {
     const int i = (threadIdx.x + e * 256) * 4;
@@ -206,17 +220,14 @@ __global__ void __launch_bounds__(256) stream_rms_vec_kernel(float* __restrict__
 #pragma unroll
       for (int u = 0; u < 4; ++u) z[u] = held[e][u] * r * g[u];
     }
-    if constexpr (FILTER) {           // both filters' old inputs are asked for before anything is stored
-      Filter4<TAPS> f1, f2;
+    if constexpr (FILTER) {
       float a[4], b[4];
-      f1.load(f.held1, slot, carried, i, dim, dt_out);
-      if (w2) f2.load(f.held2, slot, carried, i, dim, dt_out);
 #pragma unroll
       for (int u = 0; u < 4; ++u) { a[u] = rounded(y[u], dt_out); b[u] = w2 ? rounded(z[u], dt_out) : 0.f; }
-      f1.apply(a, f.w1, i, dt_out, y);
-      if (w2) f2.apply(b, f.w2, i, dt_out, z);
-      f1.keep(f.held1, a, dim, dt_out);
-      if (w2) f2.keep(f.held2, b, dim, dt_out);
+      f1[e].apply(a, y);
+      if (w2) f2[e].apply(b, z);
+      f1[e].keep(f.held1, a, dim, dt_out);
+      if (w2) f2[e].keep(f.held2, b, dim, dt_out);
     }
     store4(y1, base + i, dt_out, y);
     if (w2) store4(y2, base + i, dt_out, z);
