@@ -96,6 +96,12 @@ __device__ __forceinline__ void store4(void* p, int64_t i, int dt, const float (
     *reinterpret_cast<ushort4*>(reinterpret_cast<bf16_t*>(p) + i) = h;
   }
 }
+// The same with the element type known when the kernel is compiled (a branch on the type around every load keeps the
+// loads from being under way together).
+template <int DT>
+__device__ __forceinline__ void load4t(const void* p, int64_t i, float (&v)[4]) { load4(p, i, DT, v); }
+template <int DT>
+__device__ __forceinline__ void store4t(void* p, int64_t i, const float (&v)[4]) { store4(p, i, DT, v); }
 __device__ __forceinline__ float rounded(float v, int dt) { return dt == HOLON_F32 ? v : bf16_to_float(float_to_bf16(v)); }
 
 // What the filters of a step of single tokens need (row b is token b): the taps [dim, taps] of the two filters (the
@@ -114,20 +120,20 @@ struct Filters {
 // for a row that starts its sequence): taps added oldest first in float32, then the input, one rounding; the slot
 // then holds the last taps - 1 inputs with this one at their end. `a`: the rounded inputs of channels c0 .. c0 + 3.
 // Everything is read before anything is written (a store in between would make every later load wait for it).
-template <int TAPS>
+template <int TAPS, int DT>
 struct Filter4 {
   float old[TAPS > 1 ? TAPS - 1 : 1][4];
   float taps[TAPS][4];                                   // the four channels' taps as they lie: [channel][tap] flat
   int64_t base;
-  __device__ __forceinline__ void load(const void* held, const void* w, int slot, bool carried, int c0, int dim, int dt) {
+  __device__ __forceinline__ void load(const void* held, const void* w, int slot, bool carried, int c0, int dim) {
     base = (int64_t)slot * (TAPS - 1) * dim + c0;
 #pragma unroll
-    for (int j = 0; j + 1 < TAPS; ++j) {
-      if (carried) load4(held, base + (int64_t)j * dim, dt, old[j]);
-      else old[j][0] = old[j][1] = old[j][2] = old[j][3] = 0.f;
+    for (int j = 0; j + 1 < TAPS; ++j) {                   // (a slot that is not carried is read all the same, and
+      load4t<DT>(held, base + (int64_t)j * dim, old[j]);   // what it held counts as zeros)
+      if (!carried) old[j][0] = old[j][1] = old[j][2] = old[j][3] = 0.f;
     }
 #pragma unroll
-    for (int j = 0; j < TAPS; ++j) load4(w, (int64_t)c0 * TAPS + 4 * j, dt, taps[j]);
+    for (int j = 0; j < TAPS; ++j) load4t<DT>(w, (int64_t)c0 * TAPS + 4 * j, taps[j]);
   }
   __device__ __forceinline__ void apply(const float (&a)[4], float (&y)[4]) const {
 #pragma unroll
@@ -139,17 +145,17 @@ struct Filter4 {
       y[u] = acc + a[u];
     }
   }
-  __device__ __forceinline__ void keep(void* held, const float (&a)[4], int dim, int dt) const {
+  __device__ __forceinline__ void keep(void* held, const float (&a)[4], int dim) const {
 #pragma unroll
-    for (int j = 1; j + 1 < TAPS; ++j) store4(held, base + (int64_t)(j - 1) * dim, dt, old[j]);
-    if (TAPS > 1) store4(held, base + (int64_t)(TAPS - 2) * dim, dt, a);
+    for (int j = 1; j + 1 < TAPS; ++j) store4t<DT>(held, base + (int64_t)(j - 1) * dim, old[j]);
+    if (TAPS > 1) store4t<DT>(held, base + (int64_t)(TAPS - 2) * dim, a);
   }
 };
 
 // The same pass as stream_rms_kernel with four neighbouring values a thread and step (dim a multiple of 4, at most
 // 1024 REGS values a row, which stay in registers). FILTER: the step's rows are single tokens, and each result goes
 // through its causal filter of TAPS taps before it is stored (see `filter4`).
-template <int REGS, int TAPS>
+template <int REGS, int TAPS, int DT = HOLON_BF16>     // DT: the results' (and the filters') dtype, read when TAPS > 0
 __global__ void __launch_bounds__(256) stream_rms_vec_kernel(float* __restrict__ x32, const void* __restrict__ d1, int dt1,
                                                              const void* __restrict__ d2, int dt2,
                                                              const float* __restrict__ row, const void* __restrict__ w1,
@@ -193,7 +199,7 @@ __global__ void __launch_bounds__(256) stream_rms_vec_kernel(float* __restrict__
   if (!w1) return;
   constexpr bool FILTER = TAPS > 0;
   // the filters' old inputs and taps are asked for now, so that they arrive while the row's sum is taken
-  Filter4<FILTER ? TAPS : 1> f1[FILTER ? REGS : 1], f2[FILTER ? REGS : 1];
+  Filter4<FILTER ? TAPS : 1, DT> f1[FILTER ? REGS : 1], f2[FILTER ? REGS : 1];
   if constexpr (FILTER) {
     const int slot = f.slots[blockIdx.x];
     const bool carried = f.starts[blockIdx.x] > 0;
@@ -201,8 +207,8 @@ __global__ void __launch_bounds__(256) stream_rms_vec_kernel(float* __restrict__
     for (int e = 0; e < REGS; ++e) {
       const int i = (threadIdx.x + e * 256) * 4;
       if (i >= dim) continue;
-      f1[e].load(f.held1, f.w1, slot, carried, i, dim, dt_out);
-      if (w2) f2[e].load(f.held2, f.w2, slot, carried, i, dim, dt_out);
+      f1[e].load(f.held1, f.w1, slot, carried, i, dim);
+      if (w2) f2[e].load(f.held2, f.w2, slot, carried, i, dim);
     }
   }
   sq = block_sum_256(sq, part);
@@ -226,8 +232,8 @@ __global__ void __launch_bounds__(256) stream_rms_vec_kernel(float* __restrict__
       for (int u = 0; u < 4; ++u) { a[u] = rounded(y[u], dt_out); b[u] = w2 ? rounded(z[u], dt_out) : 0.f; }
       f1[e].apply(a, y);
       if (w2) f2[e].apply(b, z);
-      f1[e].keep(f.held1, a, dim, dt_out);
-      if (w2) f2[e].keep(f.held2, b, dim, dt_out);
+      f1[e].keep(f.held1, a, dim);
+      if (w2) f2[e].keep(f.held2, b, dim);
     }
     store4(y1, base + i, dt_out, y);
     if (w2) store4(y2, base + i, dt_out, z);
@@ -288,7 +294,15 @@ extern "C" int holon_stream_rms_filter(float* x32, const void* d1, int dt1, cons
   if (rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const Filters f{cw1, cw2, held1, held2, slots, starts, taps};
-#define SRMSF(R, K) stream_rms_vec_kernel<R, K><<<(unsigned)rows, 256, 0, s>>>(x32, d1, dt1, d2, dt2, row, w1, w2, dtw, y1, y2, dim, eps, dt_out, f)
+#define SRMSF(R, K)                                                                                                  \
+  do {                                                                                                               \
+    if (dt_out == HOLON_F32)                                                                                         \
+      stream_rms_vec_kernel<R, K, HOLON_F32><<<(unsigned)rows, 256, 0, s>>>(x32, d1, dt1, d2, dt2, row, w1, w2, dtw, \
+                                                                            y1, y2, dim, eps, dt_out, f);            \
+    else                                                                                                             \
+      stream_rms_vec_kernel<R, K, HOLON_BF16><<<(unsigned)rows, 256, 0, s>>>(x32, d1, dt1, d2, dt2, row, w1, w2,     \
+                                                                             dtw, y1, y2, dim, eps, dt_out, f);      \
+  } while (0)
 #define SRMSF_BY_TAPS(R)                                                        \
   do {                                                                          \
     if (taps == 1) SRMSF(R, 1); else if (taps == 2) SRMSF(R, 2);                \

@@ -16,7 +16,7 @@
 #include "common.h"
 #include "holon_hip.h"
 
-#define SMX_MAX_D 512
+#define SMX_MAX_D 1024
 
 namespace {
 
