@@ -1,7 +1,8 @@
 """Softmax attention over the paged cache for heads whose keys and values may differ in width, with the options a
 design may name: biases on the q/k/v projections, rotary positions in either pairing, a scale of its own, a sliding
-window, and a sink (one trained scalar for each head whose exponential is added to the softmax's normaliser; nothing
-is read from the cache for it).
+window (which may keep the first tokens of the sequence visible), a sink (one trained scalar for each head whose
+exponential is added to the softmax's normaliser; nothing is read from the cache for it), one RMS norm over a token's
+whole query or key projection, a tanh cap on the scores and a logarithmic distance bias per head.
 Two mixers use it: `attention` (grouped queries) and `latent_attention` (keys and values rebuilt from a cached
 low-rank latent, computed in the latent's space so that nothing but the latent is kept).
 
