@@ -182,17 +182,20 @@ __global__ void __launch_bounds__(256) moe_router_kernel(const T* __restrict__ x
 }
 
 // y[t, c] = round(round(silu(gate)) * up) * weight of the column's expert, 0 where that weight is 0; columns from
-// experts * ff on belong to an expert every token uses with weight 1. VEC: a thread takes 16 bytes of a row at a time
+// experts * ff on belong to an expert every token uses with weight 1, or with the weight in column `shared_col` of the
+// weights' rows (which are `wstride` long). VEC: a thread takes 16 bytes of a row at a time
 // (every row and the border between gates and ups fall on 16 bytes, and a group of columns is one expert's).
 template <typename T, bool VEC>
 __global__ void __launch_bounds__(256) moe_gate_kernel(const T* __restrict__ gate_up, const float* __restrict__ weights,
-                                                       T* __restrict__ y, int experts, int ff, int shared) {
+                                                       T* __restrict__ y, int experts, int ff, int shared,
+                                                       int wstride, int shared_col) {
   const int cols = experts * ff + shared;
   const int64_t t = blockIdx.y;
   const T* row = gate_up + t * 2 * cols;
   constexpr int N = VEC ? Elem<T>::kVec : 1;
   for (int c = (blockIdx.x * 256 + threadIdx.x) * N; c < cols; c += gridDim.x * 256 * N) {
-    const float w = c < experts * ff ? weights[t * experts + c / ff] : 1.0f;
+    const float w = c < experts * ff ? weights[t * wstride + c / ff]
+                                     : (shared_col >= 0 ? weights[t * wstride + shared_col] : 1.0f);
     if constexpr (VEC) {
       uint4 out = make_uint4(0u, 0u, 0u, 0u);
       if (w != 0.f) {
@@ -212,6 +215,83 @@ __global__ void __launch_bounds__(256) moe_gate_kernel(const T* __restrict__ gat
         out = Elem<T>::round(Elem<T>::round(silu<T>(g)) * u) * w;
       }
       y[t * cols + c] = Elem<T>::store(out);
+    }
+  }
+}
+// The other router, one block of 256 threads a token: float32 logits z_e = x . router[e] + bias[e] as above; the `top`
+// largest are chosen (equal ones: the lower index first) and weighted by the softmax over the chosen logits alone, every
+// other expert 0. Rows of `router` beyond the experts are gates: their columns hold sigmoid(x . router[r]).
+template <typename T>
+__global__ void __launch_bounds__(256) moe_router_top_kernel(const T* __restrict__ x, const float* __restrict__ router,
+                                                             const float* __restrict__ bias, float* __restrict__ weights,
+                                                             int width, int experts, int rows_r, int top) {
+  extern __shared__ float xs[];                          // [width]
+  __shared__ float z_s[ROUTE_MAX_E + 1];
+  __shared__ float e_s[ROUTE_MAX_E];
+  __shared__ float red_s[4];
+  const int64_t t = blockIdx.x;
+  for (int i = threadIdx.x; i < width; i += 256) xs[i] = Elem<T>::load(x[t * width + i]);
+  __syncthreads();
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const bool wide = width % 4 == 0 && (uintptr_t)router % 16 == 0;
+  for (int e = wave; e < rows_r; e += 4) {
+    const float* w = router + (int64_t)e * width;
+    float acc = 0.f;
+    if (wide) {
+      for (int i = lane * 4; i < width; i += WAVE * 4) {
+        const float4 v = *reinterpret_cast<const float4*>(w + i);
+        acc += xs[i] * v.x + xs[i + 1] * v.y + xs[i + 2] * v.z + xs[i + 3] * v.w;
+      }
+    } else {
+      for (int i = lane; i < width; i += WAVE) acc += xs[i] * w[i];
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) z_s[e] = e < experts ? acc + (bias ? bias[e] : 0.f) : acc;
+  }
+  __syncthreads();
+  // the largest logit is always chosen: the softmax over the chosen ones is taken about it
+  float top_z = -INFINITY;
+  for (int e = threadIdx.x; e < experts; e += 256) top_z = fmaxf(top_z, z_s[e]);
+  top_z = wave_max(top_z);
+  if (lane == 0) red_s[wave] = top_z;
+  __syncthreads();
+  top_z = fmaxf(fmaxf(red_s[0], red_s[1]), fmaxf(red_s[2], red_s[3]));
+  __syncthreads();
+  float part = 0.f;
+  for (int e = threadIdx.x; e < experts; e += 256) {
+    const float mine = z_s[e];
+    int ahead = 0;
+    for (int o = 0; o < experts; ++o) ahead += (z_s[o] > mine) || (z_s[o] == mine && o < e);
+    const float v = ahead < top ? expf(mine - top_z) : 0.f;
+    e_s[e] = v;
+    part += v;
+  }
+  part = wave_sum(part);
+  if (lane == 0) red_s[wave] = part;
+  __syncthreads();
+  const float sum = ((red_s[0] + red_s[1]) + red_s[2]) + red_s[3];
+  for (int e = threadIdx.x; e < rows_r; e += 256)
+    weights[t * rows_r + e] = e < experts ? e_s[e] / sum : 1.0f / (1.0f + expf(-z_s[e]));
+}
+
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(256) relu2_kernel(const T* __restrict__ z, T* __restrict__ y, int64_t n) {
+  constexpr int N = VEC ? Elem<T>::kVec : 1;
+  for (int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * N; i < n; i += (int64_t)gridDim.x * 256 * N) {
+    if constexpr (VEC) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(z + i);
+      const T* in = reinterpret_cast<const T*>(&raw);
+      uint4 out;
+      T* o = reinterpret_cast<T*>(&out);
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        const float v = fmaxf(Elem<T>::load(in[j]), 0.f);
+        o[j] = Elem<T>::store(v * v);
+      }
+      *reinterpret_cast<uint4*>(y + i) = out;
+    } else {
+      const float v = fmaxf(Elem<T>::load(z[i]), 0.f);
+      y[i] = Elem<T>::store(v * v);
     }
   }
 }
@@ -279,9 +359,11 @@ extern "C" int holon_moe_router(const void* x, const float* router, const float*
 }
 
 extern "C" int holon_moe_gate(const void* gate_up, const float* weights, void* y, int64_t rows, int experts, int ff,
-                              int shared, int dtype, void* stream) {
+                              int shared, int dtype, int wstride, int shared_col, void* stream) {
   HOLON_CHECK(rows >= 0 && rows <= 65535 * 1024LL && experts >= 1 && ff >= 1 && shared >= 0,
               "moe_gate: rows=%lld, %d experts of %d, %d shared columns", (long long)rows, experts, ff, shared);
+  HOLON_CHECK(wstride >= experts && shared_col < wstride, "moe_gate: weight rows of %d for %d experts, column %d",
+              wstride, experts, shared_col);
   if (rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const int cols = experts * ff + shared;
@@ -292,11 +374,50 @@ extern "C" int holon_moe_gate(const void* gate_up, const float* weights, void* y
     const int groups = wide ? cols / vec : cols;
     const dim3 grid((groups + 255) / 256 < 64 ? (groups + 255) / 256 : 64, n);
 #define MOE_GATE(T, V)                                                                                        \
-  moe_gate_kernel<T, V><<<grid, 256, 0, s>>>((const T*)gate_up + r0 * 2 * cols, weights + r0 * experts,       \
-                                             (T*)y + r0 * cols, experts, ff, shared)
+  moe_gate_kernel<T, V><<<grid, 256, 0, s>>>((const T*)gate_up + r0 * 2 * cols, weights + r0 * wstride,       \
+                                             (T*)y + r0 * cols, experts, ff, shared, wstride, shared_col)
     if (dtype == HOLON_F32) { if (wide) MOE_GATE(float, true); else MOE_GATE(float, false); }
     else { if (wide) MOE_GATE(bf16_t, true); else MOE_GATE(bf16_t, false); }
 #undef MOE_GATE
+  }
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_moe_router_top(const void* x, const float* router, const float* bias, float* weights, int64_t rows,
+                                    int width, int experts, int router_rows, int top, int dtype, void* stream) {
+  HOLON_CHECK(rows >= 0 && rows <= 0x7fffffffLL && width >= 1 && width <= 12288 && experts >= 1 &&
+                  experts <= ROUTE_MAX_E && top >= 1 && top <= experts &&
+                  (router_rows == experts || router_rows == experts + 1),
+              "moe_router_top: rows=%lld of %d (at most 12,288), top %d of %d experts (at most %d), %d router rows",
+              (long long)rows, width, top, experts, ROUTE_MAX_E, router_rows);
+  if (rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t lds = (size_t)width * sizeof(float);
+  if (dtype == HOLON_F32)
+    moe_router_top_kernel<float><<<(unsigned)rows, 256, lds, s>>>((const float*)x, router, bias, weights, width,
+                                                                 experts, router_rows, top);
+  else
+    moe_router_top_kernel<bf16_t><<<(unsigned)rows, 256, lds, s>>>((const bf16_t*)x, router, bias, weights, width,
+                                                                  experts, router_rows, top);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_relu2(const void* z, void* y, int64_t n, int dtype, void* stream) {
+  HOLON_CHECK(n >= 0, "relu2: n=%lld", (long long)n);
+  if (n == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int vec = dtype == HOLON_F32 ? 4 : 8;
+  const bool wide = n % vec == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)y % 16 == 0;
+  const int64_t groups = wide ? n / vec : n;
+  const unsigned blocks = (unsigned)((groups + 255) / 256 < 16384 ? (groups + 255) / 256 : 16384);
+  if (dtype == HOLON_F32) {
+    if (wide) relu2_kernel<float, true><<<blocks, 256, 0, s>>>((const float*)z, (float*)y, n);
+    else relu2_kernel<float, false><<<blocks, 256, 0, s>>>((const float*)z, (float*)y, n);
+  } else {
+    if (wide) relu2_kernel<bf16_t, true><<<blocks, 256, 0, s>>>((const bf16_t*)z, (bf16_t*)y, n);
+    else relu2_kernel<bf16_t, false><<<blocks, 256, 0, s>>>((const bf16_t*)z, (bf16_t*)y, n);
   }
   HOLON_LAUNCH_OK();
   return 0;

@@ -240,7 +240,8 @@ int holon_decay_lora(const float* a, const void* w2t, const float* w0, float* y,
 int holon_head_prepare(const void* qkv, void* q_out, int tokens, int heads, int kv_heads, int dim, int vdim,
                        const void* q_weight, const void* k_weight, float eps, const float* table, int rot, int table_rows,
                        const int32_t* positions, void* pages, const int32_t* write_page, const int32_t* write_off,
-                       int page_size, int num_pages, int dtype, const float* bias, void* stream);
+                       int page_size, int num_pages, int dtype, const float* bias, int stride, int v_from_keys,
+                       int v_repeat, void* stream);
 int holon_sigmoid_attention(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
                             const int32_t* slots, const int32_t* token_row, const int32_t* positions,
                             const int32_t* query_start, const int32_t* row_ids, int tokens, int heads, int kv_heads,
@@ -276,6 +277,13 @@ int holon_softmax_attention(const void* q, void* out, const void* pages, const i
                             int tokens, int heads, int kv_heads, int dim, int vdim, int page_size, int num_pages,
                             const float* sink, float scale, int window, int dtype, float softcap, const float* r1,
                             const float* r2, int keep_first, void* stream);
+// x [T, H V] *= sigmoid(gates[t, h]) per head (gates: columns of rows gate_stride apart); x [rows, dim] += bias;
+// y [T, 2 H V] (kv head, map, head in group) -> out [T, H V]: u = y1 - lam y2, u / sqrt(mean(u^2) + eps) * gain.
+int holon_head_gate(void* x, const void* gates, int64_t gate_stride, int64_t tokens, int heads, int vdim, int dtype,
+                    void* stream);
+int holon_add_bias(void* x, const float* bias, int64_t rows, int dim, int dtype, void* stream);
+int holon_diff_combine(const void* y, void* out, int64_t tokens, int heads, int kv_heads, int vdim, float lam, float eps,
+                       float gain, int dtype, void* stream);
 // qkv [T, H D + G D + G V]: the query values of a token RMS-normed as one vector with q_weight [H D], its key values
 // with k_weight [G D]; queries to q [T, H, D], keys and values into the token's page.
 int holon_whole_norm_prepare(const void* qkv, int tokens, int heads, int kv_heads, int dim, int vdim,
@@ -332,9 +340,17 @@ int holon_moe_route(const float* logits, const float* correction, float* weights
 int holon_moe_router(const void* x, const float* router, const float* correction, float* weights, int64_t rows,
                      int width, int experts, int top, int groups, int keep, float scale, int dtype, void* stream);
 // gate_up [rows, 2 C], C = experts ff + shared: y [rows, C] = silu(gate) up times the weight of the column's expert
-// (the last `shared` columns: 1), exactly 0 where the weight is 0.
+// (the last `shared` columns: 1, or column `shared_col` >= 0 of the weights' rows), exactly 0 where the weight is 0.
+// A row of `weights` is `wstride` long.
 int holon_moe_gate(const void* gate_up, const float* weights, void* y, int64_t rows, int experts, int ff, int shared,
-                   int dtype, void* stream);
+                   int dtype, int wstride, int shared_col, void* stream);
+// The other router: logits x . router[e] + bias[e] (nullable), the `top` largest chosen, weights the softmax over the
+// chosen logits alone; router rows beyond the experts (none or one) are gates: their columns hold a sigmoid.
+// weights [rows, router_rows].
+int holon_moe_router_top(const void* x, const float* router, const float* bias, float* weights, int64_t rows, int width,
+                         int experts, int router_rows, int top, int dtype, void* stream);
+// y = max(z, 0)^2 over n values.
+int holon_relu2(const void* z, void* y, int64_t n, int dtype, void* stream);
 
 // -- the matrix memory of xLSTM (mlstm.hip) -------------------------------------------------------------------------------
 // proj [T, width]: q, k [H D] and v [H V] and the gates' pre-activations [2 H] (input, then forget) from the given

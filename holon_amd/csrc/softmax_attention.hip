@@ -417,6 +417,50 @@ __global__ void __launch_bounds__(256) latent_rope_prepare_kernel(
     vals[(int64_t)d * page_size + off] = e;
   }
 }
+// x[t, h, :] *= sigmoid(gates[t, h]): one wave a (token, head); the gates are columns of rows `gate_stride` apart.
+template <typename T>
+__global__ void __launch_bounds__(256) head_gate_kernel(T* __restrict__ x, const T* __restrict__ gates,
+                                                        int64_t gate_stride, int64_t pairs, int heads, int vdim) {
+  const int64_t at = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
+  if (at >= pairs) return;
+  const int lane = threadIdx.x % WAVE;
+  const int64_t t = at / heads;
+  const int h = (int)(at % heads);
+  const float g = 1.0f / (1.0f + expf(-Elem<T>::load(gates[t * gate_stride + h])));
+  T* row = x + at * vdim;
+  for (int d = lane; d < vdim; d += WAVE) row[d] = Elem<T>::store(Elem<T>::load(row[d]) * g);
+}
+
+// x[t, :] += bias: the sum in float32, one rounding.
+template <typename T>
+__global__ void __launch_bounds__(256) add_bias_kernel(T* __restrict__ x, const float* __restrict__ bias, int dim) {
+  T* row = x + (int64_t)blockIdx.x * dim;
+  for (int d = threadIdx.x; d < dim; d += 256) row[d] = Elem<T>::store(Elem<T>::load(row[d]) + bias[d]);
+}
+
+// Two maps' results to one: y [T, G, 2, R, V] (kv head, map, head within the group) -> out [T, G, R, V]:
+// u = y1 - lam y2, u / sqrt(mean(u^2) + eps) * gain over a head's V values. One wave a (token, head).
+template <typename T>
+__global__ void __launch_bounds__(256) diff_combine_kernel(const T* __restrict__ y, T* __restrict__ out, int64_t pairs,
+                                                           int heads, int group, int vdim, float lam, float eps,
+                                                           float gain) {
+  const int64_t at = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
+  if (at >= pairs) return;
+  const int lane = threadIdx.x % WAVE;
+  const int64_t t = at / heads;
+  const int h = (int)(at % heads), g = h / group, j = h % group;
+  const T* first = y + ((t * 2 * heads) + (int64_t)(g * 2) * group + j) * vdim;
+  const T* second = first + (int64_t)group * vdim;
+  float ss = 0.f;
+  for (int d = lane; d < vdim; d += WAVE) {
+    const float u = Elem<T>::load(first[d]) - lam * Elem<T>::load(second[d]);
+    ss += u * u;
+  }
+  const float r = gain / sqrtf(wave_sum(ss) / (float)vdim + eps);
+  T* dst = out + at * vdim;
+  for (int d = lane; d < vdim; d += WAVE)
+    dst[d] = Elem<T>::store((Elem<T>::load(first[d]) - lam * Elem<T>::load(second[d])) * r);
+}
 }  // namespace
 
 extern "C" int holon_whole_norm_prepare(const void* qkv, int tokens, int heads, int kv_heads, int dim, int vdim,
@@ -462,6 +506,52 @@ extern "C" int holon_latent_rope_prepare(const void* both, int tokens, int heads
                                                              (const bf16_t*)c_weight, eps, table, rd, table_rows,
                                                              positions, (bf16_t*)qn, (bf16_t*)full, (bf16_t*)pages,
                                                              write_page, write_off, page_size, num_pages);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_head_gate(void* x, const void* gates, int64_t gate_stride, int64_t tokens, int heads, int vdim,
+                               int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && heads > 0 && vdim > 0 && gate_stride >= heads && tokens * heads <= 4LL * 0x7fffffff,
+              "head_gate: %lld tokens, %d heads of %d, gates %lld apart", (long long)tokens, heads, vdim,
+              (long long)gate_stride);
+  if (tokens == 0) return 0;
+  const int64_t pairs = tokens * heads;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HOLON_F32)
+    head_gate_kernel<float><<<(unsigned)((pairs + 3) / 4), 256, 0, s>>>((float*)x, (const float*)gates, gate_stride,
+                                                                        pairs, heads, vdim);
+  else
+    head_gate_kernel<bf16_t><<<(unsigned)((pairs + 3) / 4), 256, 0, s>>>((bf16_t*)x, (const bf16_t*)gates, gate_stride,
+                                                                         pairs, heads, vdim);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_add_bias(void* x, const float* bias, int64_t rows, int dim, int dtype, void* stream) {
+  HOLON_CHECK(rows >= 0 && rows <= 0x7fffffffLL && dim > 0, "add_bias: rows=%lld dim=%d", (long long)rows, dim);
+  if (rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HOLON_F32) add_bias_kernel<float><<<(unsigned)rows, 256, 0, s>>>((float*)x, bias, dim);
+  else add_bias_kernel<bf16_t><<<(unsigned)rows, 256, 0, s>>>((bf16_t*)x, bias, dim);
+  HOLON_LAUNCH_OK();
+  return 0;
+}
+
+extern "C" int holon_diff_combine(const void* y, void* out, int64_t tokens, int heads, int kv_heads, int vdim, float lam,
+                                  float eps, float gain, int dtype, void* stream) {
+  HOLON_CHECK(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && vdim > 0 &&
+                  tokens * heads <= 4LL * 0x7fffffff,
+              "diff_combine: %lld tokens, %d/%d heads of %d", (long long)tokens, heads, kv_heads, vdim);
+  if (tokens == 0) return 0;
+  const int64_t pairs = tokens * heads;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HOLON_F32)
+    diff_combine_kernel<float><<<(unsigned)((pairs + 3) / 4), 256, 0, s>>>((const float*)y, (float*)out, pairs, heads,
+                                                                           heads / kv_heads, vdim, lam, eps, gain);
+  else
+    diff_combine_kernel<bf16_t><<<(unsigned)((pairs + 3) / 4), 256, 0, s>>>((const bf16_t*)y, (bf16_t*)out, pairs, heads,
+                                                                            heads / kv_heads, vdim, lam, eps, gain);
   HOLON_LAUNCH_OK();
   return 0;
 }

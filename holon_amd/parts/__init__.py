@@ -3,7 +3,7 @@ from .base import (FLOAT32, INT32, MODEL, Build, EmbedPart, NormPart, PagedState
                    Stream)
 from .blocks import PreNorm
 from .embed import Embedding, LMHead
-from .ffn import MoE, PolyNormFFN, SwiGLU
+from .ffn import DenseFFN, MoE, PolyNormFFN, SwiGLU
 from .linear import Linear
 from .mixers import GQA, ParallelMixers
 from .norms import Normed, RMSNorm
@@ -15,10 +15,11 @@ from .stream32 import LayerNorm, Pending, PreNorm32
 from .dyt import DynamicTanh, Sandwich32, Scaled
 from .softmax_attention import LatentAttention, SoftmaxAttention
 from .mlstm import MLSTM
+from .diff_attention import DiffAttention
 from .parallel_block import Parallel32, RMSNorm32
 
 __all__ = ["FLOAT32", "INT32", "MODEL", "Build", "EmbedPart", "NormPart", "PagedState", "ParamDecl", "Part", "PartialSums", "SlotState", "Stream", "PreNorm",
            "Embedding", "LMHead", "SwiGLU", "Linear", "GQA", "Normed", "RMSNorm", "NoPosition", "Rope", "rope_table", "BandedRope", "CausalConv", "DecayMemory", "GatedDelta",
            "SigmoidWindowAttention", "LayerNorm", "Pending", "PreNorm32", "ParallelMixers",
            "DynamicTanh", "Sandwich32", "Scaled", "LatentAttention", "SoftmaxAttention", "MLSTM", "YarnRope",
-           "MoE", "PolyNormFFN", "Parallel32", "RMSNorm32"]
+           "MoE", "PolyNormFFN", "Parallel32", "RMSNorm32", "DiffAttention", "DenseFFN"]

@@ -138,30 +138,72 @@ def _moe_router_hip(launch, x, router, correction, top, groups, keep, scale):
     return weights
 
 
-def moe_gate_plain(gate_up, weights, ff, shared):
+def moe_gate_plain(gate_up, weights, ff, shared, shared_weight=False):
     """gate_up [T, 2 C] with C = E ff + shared columns of gates, then as many of ups; weights [T, E] float32.
     -> [T, C]: silu(gate) * up (as `silu_mul` rounds it), times the weight of the column's expert (column c belongs to
     expert c // ff; the last `shared` columns to an expert that every token uses with weight 1); exactly 0 where the
-    weight is 0. One more rounding for the weight."""
-    t, e = weights.shape
+    weight is 0. One more rounding for the weight. `shared_weight`: weights is [T, E + 1] and its last column is the
+    weight of the shared expert's columns."""
+    t, e = weights.shape[0], weights.shape[1] - int(bool(shared_weight))
     c = e * ff + shared
     g, u = gate_up[:, :c].float(), gate_up[:, c:].float()
     act = ((g * torch.sigmoid(g)).to(gate_up.dtype).float() * u).to(gate_up.dtype)
-    w = weights.repeat_interleave(ff, dim=1)
+    w = weights[:, :e].repeat_interleave(ff, dim=1)
     if shared:
-        w = torch.cat((w, torch.ones((t, shared), dtype=w.dtype, device=w.device)), dim=1)
+        last = weights[:, e:].expand(t, shared) if shared_weight else torch.ones((t, shared), dtype=w.dtype, device=w.device)
+        w = torch.cat((w, last), dim=1)
     return torch.where(w == 0, torch.zeros_like(act), (act.float() * w).to(gate_up.dtype))
 
 
-def _moe_gate_hip(launch, gate_up, weights, ff, shared):
-    t, e = weights.shape
+def _moe_gate_hip(launch, gate_up, weights, ff, shared, shared_weight=False):
+    t, e = weights.shape[0], weights.shape[1] - int(bool(shared_weight))
     c = e * ff + shared
     _need(gate_up.is_cuda and gate_up.is_contiguous() and gate_up.dtype in _DT and gate_up.shape == (t, 2 * c)
-          and weights.is_contiguous() and weights.dtype == torch.float32,
+          and weights.is_contiguous() and weights.dtype == torch.float32 and e >= 1,
           f"moe_gate: rows {tuple(gate_up.shape)} for {e} experts of {ff} and {shared} shared columns")
     y = torch.empty((t, c), dtype=gate_up.dtype, device=gate_up.device)
     if t:
-        launch(gate_up.data_ptr(), weights.data_ptr(), y.data_ptr(), t, e, ff, shared, _DT[gate_up.dtype])
+        launch(gate_up.data_ptr(), weights.data_ptr(), y.data_ptr(), t, e, ff, shared, _DT[gate_up.dtype],
+               weights.shape[1], e if shared_weight else -1)
+    return y
+
+
+def moe_router_top_plain(x, router, bias, experts, top):
+    """x [T, W] (any dtype), router [R, W] float32 with R = experts or experts + 1, bias [experts] float32 or None:
+    the float32 logits z = x . router[e] + bias[e]; the `top` largest are chosen (equal ones: the lower index first)
+    and weighted by the softmax over the chosen logits alone, every other expert 0. A last row beyond the experts is a
+    gate: its column holds sigmoid(x . router[experts]). -> [T, R] float32."""
+    z = x.float() @ router.float().T
+    logits = z[:, :experts] + (bias.float() if bias is not None else 0.0)
+    order = torch.sort(logits, dim=-1, descending=True, stable=True).indices[:, :top]
+    chosen = logits.gather(1, order)
+    w = torch.zeros_like(logits).scatter_(1, order, torch.softmax(chosen, dim=-1))
+    return torch.cat((w, torch.sigmoid(z[:, experts:])), dim=1).contiguous()
+
+
+def _moe_router_top_hip(launch, x, router, bias, experts, top):
+    (t, w), r = x.shape, router.shape[0]
+    _need(x.is_cuda and x.is_contiguous() and x.dtype in _DT and router.is_contiguous() and router.dtype == torch.float32
+          and router.shape == (r, w) and r in (experts, experts + 1) and 1 <= top <= experts <= 1024 and w <= 12288
+          and (bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.shape == (experts,))),
+          f"moe_router_top: rows {tuple(x.shape)} {x.dtype}, router {tuple(router.shape)}, top {top} of {experts}")
+    weights = torch.empty((t, r), dtype=torch.float32, device=x.device)
+    if t:
+        launch(x.data_ptr(), router.data_ptr(), None if bias is None else bias.data_ptr(), weights.data_ptr(), t, w,
+               experts, r, int(top), _DT[x.dtype])
+    return weights
+
+
+def relu2_plain(z):
+    """z [T, F] -> max(z, 0)^2, float32 inside, one rounding."""
+    return torch.relu(z.float()).pow(2).to(z.dtype)
+
+
+def _relu2_hip(launch, z):
+    _need(z.is_cuda and z.is_contiguous() and z.dtype in _DT, "relu2: contiguous float32 or bfloat16 values on the GPU")
+    y = torch.empty_like(z)
+    if z.numel():
+        launch(z.data_ptr(), y.data_ptr(), z.numel(), _DT[z.dtype])
     return y
 
 
@@ -170,7 +212,11 @@ register_kernel(KernelOp("moe_route", moe_route_plain, "holon_moe_route", [_P, _
                          _moe_route_hip))
 register_kernel(KernelOp("moe_router", moe_router_plain, "holon_moe_router",
                          [_P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _F, _I], _moe_router_hip))
-register_kernel(KernelOp("moe_gate", moe_gate_plain, "holon_moe_gate", [_P, _P, _P, _L, _I, _I, _I, _I], _moe_gate_hip))
+register_kernel(KernelOp("moe_gate", moe_gate_plain, "holon_moe_gate", [_P, _P, _P, _L, _I, _I, _I, _I, _I, _I],
+                         _moe_gate_hip))
+register_kernel(KernelOp("moe_router_top", moe_router_top_plain, "holon_moe_router_top",
+                         [_P, _P, _P, _P, _L, _I, _I, _I, _I, _I], _moe_router_top_hip))
+register_kernel(KernelOp("relu2", relu2_plain, "holon_relu2", [_P, _P, _L, _I], _relu2_hip))
 
 
 @register_part("ffn", "polynorm")
@@ -193,9 +239,35 @@ class PolyNormFFN(Part):
     __call__ = forward
 
 
+@register_part("ffn", "dense")
+class DenseFFN(Part):
+    """down(act(up(x))) with an activation by name: `relu2`, the square of max(z, 0)."""
+
+    graph_safe = True
+    ACTS = ("relu2",)
+
+    def __init__(self, build: Build, *, inter: int, hidden: int, layer: int, act: str = "relu2") -> None:
+        super().__init__(build)
+        if act not in self.ACTS:
+            raise ValueError(f"ffn dense: no activation {act!r} ({', '.join(self.ACTS)})")
+        self.inter, self.hidden, self.act = inter, hidden, act
+        self.attach("up_proj", Linear(build, inp=hidden, out=inter))
+        self.attach("down_proj", Linear(build, inp=inter, out=hidden))
+
+    def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
+        return self.down_proj(self.kernels.relu2(self.up_proj(x)))
+
+    __call__ = forward
+
+
 @register_part("ffn", "moe")
 class MoE(Part):
-    """A mixture of SiLU-gated experts with a sigmoid router, and an optional shared expert that every token uses.
+    """A mixture of SiLU-gated experts with a router, and an optional shared expert that every token uses.
+
+    `score` "softmax_top" is the other router: float32 logits z = W_r x + b (`router_bias`), the `top` largest z are
+    chosen and weighted by the softmax over the chosen z alone (no groups, no scale). `shared_gated`: the shared
+    expert's output is multiplied by sigmoid(w_sg . x), one number a token; w_sg rides as one more row of the router's
+    weights, so the router's kernel leaves that weight too. What follows describes `score` "sigmoid".
 
     Router: float32 logits (products of the input as it is with float32 weights, summed in float32), scores s =
     sigmoid(logits); experts are chosen by s + `correction` (`bias`), optionally
@@ -208,10 +280,18 @@ class MoE(Part):
     graph_safe = True
 
     def __init__(self, build: Build, *, experts: int, top: int, inter: int, hidden: int, layer: int,
-                 scale: float = 1.0, groups: int = 1, keep: int = 1, bias: bool = True, shared: int = 0) -> None:
+                 scale: float = 1.0, groups: int = 1, keep: int = 1, bias: bool = True, shared: int = 0,
+                 score: str = "sigmoid", shared_gated: bool = False) -> None:
         super().__init__(build)
         if not 1 <= top <= experts:
             raise ValueError(f"moe: top {top} of {experts} experts")
+        if score not in ("sigmoid", "softmax_top"):
+            raise ValueError(f"moe: no router score {score!r} (sigmoid, softmax_top)")
+        if score == "softmax_top" and (groups > 1 or float(scale) != 1.0):
+            raise ValueError("moe: the softmax over the chosen logits comes without groups and without a scale")
+        if shared_gated and (not shared or score != "softmax_top"):
+            raise ValueError("moe: a gate on the shared expert needs a shared expert and the softmax_top router")
+        self.score, self.shared_gated = score, bool(shared_gated)
         if groups > 1 and (experts % groups or not 1 <= keep <= groups or top > keep * (experts // groups)):
             raise ValueError(f"moe: {experts} experts in {groups} groups, {keep} kept, top {top}")
         self.experts, self.top, self.inter, self.hidden, self.shared = experts, top, inter, hidden, int(shared)
@@ -219,7 +299,10 @@ class MoE(Part):
         self.declare("router", (experts, hidden), kind=FLOAT32)
         self.has_bias = bool(bias)
         if self.has_bias:
-            self.declare("correction", (experts,), kind=FLOAT32, init="zero")
+            # (sigmoid: a correction of the choice alone; softmax_top: the logits' bias)
+            self.declare("correction" if score == "sigmoid" else "router_bias", (experts,), kind=FLOAT32, init="zero")
+        if self.shared_gated:
+            self.declare("shared_sg", (1, hidden), kind=FLOAT32)
         self.declare("gate", (experts, inter, hidden))
         self.declare("up", (experts, inter, hidden))
         self.declare("down", (experts, hidden, inter))
@@ -233,6 +316,10 @@ class MoE(Part):
     def finalize(self) -> None:
         if self.gate is None:
             return
+        if self.shared_gated and self.router.shape[0] == self.experts:
+            self.router = torch.cat((self.router, self.shared_sg)).contiguous()
+            del self._decls["shared_sg"]
+            self.shared_sg = None
         e, f, w = self.experts, self.inter, self.hidden
         cols = e * f + self.shared
         gate_up, down = Linear(self.build, inp=w, out=2 * cols), Linear(self.build, inp=cols, out=w)
@@ -255,6 +342,11 @@ class MoE(Part):
 
     def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
         k = self.kernels
+        if self.score == "softmax_top":
+            weights = k.moe_router_top(x, self.router, self.router_bias if self.has_bias else None, self.experts,
+                                       self.top)
+            act = k.moe_gate(self.gate_up(x), weights, self.inter, self.shared, shared_weight=self.shared_gated)
+            return self.all_down(act)
         weights = k.moe_router(x, self.router, self.correction if self.has_bias else None, self.top, self.groups,
                                self.keep, self.scale)
         act = k.moe_gate(self.gate_up(x), weights, self.inter, self.shared)

@@ -8,7 +8,11 @@ Both norms are RMS norms of the same rows, so they share the row's mean square a
 vector of the pass that begins (`pass_steps`: a tensor `[passes, hidden]` whose row `site.turn` is added in front of
 every pass, the first too). f1 and f2 (`conv_taps` > 0) replace a sublayer's input a by a + conv(a), a short causal
 filter over time on every channel whose last taps - 1 inputs are part of the request's state. A layer may lack the
-feed-forward; its second norm and filter are then not built.
+feed-forward; its second norm and filter are then not built. With `shared_norm` the block has one norm and both
+sublayers read its result: x += mixer(f1(norm1(x))) + ffn(f1(norm1(x))).
+
+The norm `rms32` may hold its weight around zero (`one_plus`): y = x / sqrt(mean(x^2) + eps) * (1 + w); the sum 1 + w is
+formed once after loading, in float32, and kept in float32 whatever the engine's dtype.
 """
 from __future__ import annotations
 
@@ -152,14 +156,24 @@ register_kernel(KernelOp("scale_rows", scale_rows_plain, "holon_scale_rows", [_P
 @register_part("norm", "rms32")
 class RMSNorm32(NormPart):
     """y = x * rsqrt(mean(x^2) + eps) * weight over rows of a float32 stream (rows in the engine's dtype are widened
-    first); float32 inside, the result in the engine's dtype."""
+    first); float32 inside, the result in the engine's dtype. `one_plus`: the stored weight w lies around zero and the
+    norm multiplies by 1 + w (kept in float32: in bfloat16 the sum would lose what w holds)."""
 
     graph_safe = True
 
-    def __init__(self, build: Build, *, eps: float, dim: int) -> None:
+    def __init__(self, build: Build, *, eps: float, dim: int, one_plus: bool = False) -> None:
         super().__init__(build)
-        self.eps, self.dim = float(eps), dim
-        self.declare("weight", (dim,), init="norm")
+        self.eps, self.dim, self.one_plus = float(eps), dim, bool(one_plus)
+        if self.one_plus:
+            self.declare("weight", (dim,), kind=FLOAT32, init="tap")
+        else:
+            self.declare("weight", (dim,), init="norm")
+        self._summed = False
+
+    def finalize(self) -> None:
+        if self.one_plus and self.weight is not None and not self._summed:
+            self.weight = (self.weight.float() + 1.0).contiguous()
+            self._summed = True
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if x.dtype != torch.float32:
@@ -186,18 +200,20 @@ class Parallel32(Part):
     graph_safe = True
 
     def __init__(self, build: Build, *, layer: int, hidden: int, mixer: PartRef, ffn: PartRef | None, norm: PartRef,
-                 conv_taps: int = 0, pass_steps: int = 0) -> None:
+                 conv_taps: int = 0, pass_steps: int = 0, shared_norm: bool = False) -> None:
         super().__init__(build)
         self.hidden = hidden
+        self.shared_norm = bool(shared_norm)
         self.attach("norm1", build.make(norm, dim=hidden))
         self.attach("mixer", build.make(mixer, layer=layer, hidden=hidden))
         self.conv1 = self.conv2 = self.ffn = self.norm2 = None
         if conv_taps > 0:
             self.attach("conv1", CausalConv(build, channels=hidden, taps=conv_taps, add_input=True, name="filter1"))
         if ffn is not None:
-            self.attach("norm2", build.make(norm, dim=hidden))
+            if not self.shared_norm:
+                self.attach("norm2", build.make(norm, dim=hidden))
             self.attach("ffn", build.make(ffn, layer=layer, hidden=hidden))
-            if conv_taps > 0:
+            if conv_taps > 0 and not self.shared_norm:
                 self.attach("conv2", CausalConv(build, channels=hidden, taps=conv_taps, add_input=True, name="filter2"))
         self.passes = int(pass_steps)
         if self.passes > 0:
@@ -212,6 +228,7 @@ class Parallel32(Part):
             self._one_kernel = float(specs[0]["eps"])
             # (the kernel serves widths that are a multiple of 4 up to 8,192 and up to four taps; the plain form any)
             self._fused_filter = self.conv1 is not None and (self.ffn is None or self.conv2 is not None) \
+                and not self.shared_norm \
                 and self.hidden % 4 == 0 and self.hidden <= 8192 and self.conv1.taps <= 4
 
     def state(self):
@@ -254,10 +271,10 @@ class Parallel32(Part):
         return stream
 
     def _mix(self, a, b, step, site) -> list[torch.Tensor]:
-        """Both sublayers' results from their inputs."""
+        """Both sublayers' results from their inputs (one input for both under `shared_norm`)."""
         out = [self.mixer(a, step, site)]
         if self.ffn is not None:
-            out.append(self.ffn(b, step))
+            out.append(self.ffn(a if self.shared_norm else b, step))
         return out
 
     __call__ = forward

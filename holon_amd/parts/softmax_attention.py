@@ -21,7 +21,7 @@ from ..spec import PartRef
 from .base import FLOAT32, Build, PagedState, Part
 from .linear import Linear
 
-_P, _I, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+_P, _I, _L, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
 
@@ -253,6 +253,41 @@ def _latent_prepare_hip(launch, both, q_rank, q_weight, c_weight, eps, pages, wr
     return cq
 
 
+def head_gate_plain(x, gates, heads):
+    """x [T, H V], updated in place: head h of token t is multiplied by sigmoid(gates[t, h]); `gates` [T, H] may be
+    columns of wider rows (a view with a row stride). float32 inside, one rounding."""
+    t = x.shape[0]
+    v = x.view(t, heads, -1)
+    v.copy_((v.float() * torch.sigmoid(gates.float())[:, :, None]).to(x.dtype))
+    return x
+
+
+def _head_gate_hip(launch, x, gates, heads):
+    t = x.shape[0]
+    if not (x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.dtype in _DT and x.shape[1] % heads == 0
+            and gates.dtype == x.dtype and gates.shape == (t, heads) and gates.stride(1) == 1):
+        raise ValueError(f"head_gate: rows {tuple(x.shape)} {x.dtype} and gates {tuple(gates.shape)} {gates.dtype} "
+                         f"(strides {gates.stride()}) do not fit {heads} heads")
+    if t:
+        launch(x.data_ptr(), gates.data_ptr(), gates.stride(0), t, heads, x.shape[1] // heads, _DT[x.dtype])
+    return x
+
+
+def add_bias_plain(x, bias):
+    """x [T, N] += bias [N] (float32) in place: the sum in float32, one rounding."""
+    x.copy_((x.float() + bias.float()).to(x.dtype))
+    return x
+
+
+def _add_bias_hip(launch, x, bias):
+    if not (x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.dtype in _DT and bias.is_contiguous()
+            and bias.dtype == torch.float32 and bias.shape == (x.shape[1],)):
+        raise ValueError(f"add_bias: rows {tuple(x.shape)} {x.dtype} and a bias {tuple(bias.shape)} {bias.dtype}")
+    if x.shape[0]:
+        launch(x.data_ptr(), bias.data_ptr(), x.shape[0], x.shape[1], _DT[x.dtype])
+    return x
+
+
 register_kernel(KernelOp("softmax_attention", softmax_attention_plain, "holon_softmax_attention",
                          [_P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _I, _F, _P, _P, _I],
                          _softmax_attention_hip))
@@ -265,6 +300,8 @@ register_kernel(KernelOp("latent_rope_prepare", latent_rope_prepare_plain, "holo
                          _latent_rope_prepare_hip))
 register_kernel(KernelOp("latent_prepare", latent_prepare_plain, "holon_latent_prepare",
                          [_P, _I, _I, _I, _P, _P, _F, _P, _P, _P, _P, _I, _I, _I], _latent_prepare_hip))
+register_kernel(KernelOp("head_gate", head_gate_plain, "holon_head_gate", [_P, _P, _L, _L, _I, _I, _I], _head_gate_hip))
+register_kernel(KernelOp("add_bias", add_bias_plain, "holon_add_bias", [_P, _P, _L, _I, _I], _add_bias_hip))
 
 
 def attend(k, q, held, view, step, kv_heads, vdim, sink, scale, window, softcap=0.0, dist=None, keep_first=0):
@@ -300,17 +337,34 @@ class SoftmaxAttention(Part):
     are split into heads, with a weight `q_norm` of that length, and its key values likewise (`k_norm`); `softcap`:
     scores become softcap tanh(score / softcap); `distance_bias`: r1_h ln(1 + r2_h (i - j)) is taken off the score of
     key j for query i (`r1`, `r2`, one number a head each); `keep_first`: under a window the first tokens of the
-    sequence stay visible, at their true positions."""
+    sequence stay visible, at their true positions.
+
+    `values_from_keys`: there is no value projection; a token's values are its keys as projected (bias added, before
+    the rotation), so vdim = dim, and the cache holds the turned key and the unturned one side by side. `sink_value`
+    (a number): a sink that every head shares and no tensor holds (0: one is added to the softmax's denominator).
+    `head_gate`: a projection `g` of one number a head, computed with q and k in the merged product; head h's result
+    is multiplied by sigmoid(g_h) before the output projection. `o_bias`: a bias on the output projection."""
 
     graph_safe = True
 
     def __init__(self, build: Build, *, heads: int, kv_heads: int, dim: int, vdim: int, hidden: int, layer: int,
                  scale: float | None = None, window: int = 0, qkv_bias: bool = False, sink: bool = False,
                  position: PartRef | None = None, name: str = "", whole_norm: float | None = None,
-                 softcap: float = 0.0, distance_bias: bool = False, keep_first: int = 0) -> None:
+                 softcap: float = 0.0, distance_bias: bool = False, keep_first: int = 0,
+                 values_from_keys: bool = False, sink_value: float | None = None, head_gate: bool = False,
+                 o_bias: bool = False) -> None:
         super().__init__(build)
         if heads % kv_heads:
             raise ValueError(f"attention: {heads} heads are not a multiple of {kv_heads} kv heads")
+        self.values_from_keys = bool(values_from_keys)
+        if self.values_from_keys and vdim != dim:
+            raise ValueError(f"attention: values that are the keys are as wide as the keys ({dim}), not {vdim}")
+        if self.values_from_keys and whole_norm is not None:
+            raise ValueError("attention: values from the keys come without the norm over the whole projection")
+        if sink and sink_value is not None:
+            raise ValueError("attention: either a sink per head or one number for all")
+        if head_gate and whole_norm is not None:
+            raise ValueError("attention: the gate per head comes without the norm over the whole projection")
         self.heads, self.kv_heads, self.dim, self.vdim, self.hidden = heads, kv_heads, dim, vdim, hidden
         self.window = int(window)
         self.keep_first = int(keep_first) if self.window > 0 else 0
@@ -329,21 +383,32 @@ class SoftmaxAttention(Part):
         self.state_name = f"{name}.kv" if name else "kv"
         self.attach("q", Linear(build, inp=hidden, out=heads * dim))
         self.attach("k", Linear(build, inp=hidden, out=kv_heads * dim))
-        self.attach("v", Linear(build, inp=hidden, out=kv_heads * vdim))
+        if not self.values_from_keys:
+            self.attach("v", Linear(build, inp=hidden, out=kv_heads * vdim))
+        self.has_gate = bool(head_gate)
+        if self.has_gate:
+            self.attach("g", Linear(build, inp=hidden, out=heads))
         self.attach("o", Linear(build, inp=heads * vdim, out=hidden))
         self.qkv_bias = bool(qkv_bias)
         if self.qkv_bias:
             self.declare("q_bias", (heads * dim,), kind=FLOAT32, init="zero")
             self.declare("k_bias", (kv_heads * dim,), kind=FLOAT32, init="zero")
-            self.declare("v_bias", (kv_heads * vdim,), kind=FLOAT32, init="zero")
+            if not self.values_from_keys:
+                self.declare("v_bias", (kv_heads * vdim,), kind=FLOAT32, init="zero")
+        self.has_o_bias = bool(o_bias)
+        if self.has_o_bias:
+            self.declare("o_bias", (hidden,), kind=FLOAT32, init="zero")
         self.has_sink = bool(sink)
         if self.has_sink:
             self.declare("sink", (heads,), kind=FLOAT32, init="zero")
+        self.sink_value = None if sink_value is None else float(sink_value)
         self.position = None
         if position is not None:
             self.attach("position", build.make(position, head_dim=dim))
         self.qkv: Linear | None = None
         self.bias: torch.Tensor | None = None
+        self.fixed_sink: torch.Tensor | None = None
+        self.qkv_width = (heads + kv_heads) * dim + (0 if self.values_from_keys else kv_heads * vdim)
 
     def state(self):
         return [PagedState(self.state_name, elems=self.kv_heads * (self.dim + self.vdim), window=self.window,
@@ -358,31 +423,46 @@ class SoftmaxAttention(Part):
                 if self.qkv_bias:
                     setattr(self, bias, getattr(self, bias).index_select(0, order).contiguous())
         if self.qkv_bias and self.q_bias is not None:
-            self.bias = torch.cat((self.q_bias, self.k_bias, self.v_bias)).contiguous()
-        self.qkv = Linear.merge(self.build, self.q, self.k, self.v)
-        for name in ("q", "k", "v"):
+            self.bias = torch.cat([self.q_bias, self.k_bias] + ([] if self.values_from_keys else [self.v_bias])
+                                  ).contiguous()
+        if self.sink_value is not None and self.build.device.type != "meta":
+            self.fixed_sink = torch.full((self.heads,), self.sink_value, dtype=torch.float32, device=self.build.device)
+        merged = ["q", "k"] + ([] if self.values_from_keys else ["v"]) + (["g"] if self.has_gate else [])
+        if self.has_gate and self.g.weight is not None and self.heads % 16:
+            # the gates' columns are padded with rows of zeros to a multiple of 16: every product of the framework
+            # then serves the merged projection
+            pad = 16 - self.heads % 16
+            self.g.weight = torch.cat((self.g.weight, self.g.weight.new_zeros((pad, self.hidden)))).contiguous()
+            self.g.out += pad
+        self.qkv = Linear.merge(self.build, *(getattr(self, name) for name in merged))
+        for name in merged:
             self.drop(name)
         self._children["qkv"] = self.qkv
 
     def extra_tensors(self):
-        return [self.bias] if self.bias is not None else []
+        return [t for t in (self.bias, self.fixed_sink) if t is not None]
 
     def forward(self, x: torch.Tensor, step, site) -> torch.Tensor:
         k = self.kernels
         held = site.paged[self.state_name]
         view = step.paged[held.group]
         table = getattr(self.position, "table", None)
+        qkv = self.qkv(x)
         if self.whole_norm is not None:
-            q = k.whole_norm_prepare(self.qkv(x), self.heads, self.kv_heads, self.dim, self.vdim, self.q_norm,
+            q = k.whole_norm_prepare(qkv, self.heads, self.kv_heads, self.dim, self.vdim, self.q_norm,
                                      self.k_norm, self.whole_norm, held.pages, view.write_page, view.write_off,
                                      view.page_size)
         else:
-            q = k.head_prepare(self.qkv(x), self.heads, self.kv_heads, self.dim, self.vdim, None, None, 0.0, table,
+            q = k.head_prepare(qkv, self.heads, self.kv_heads, self.dim, self.vdim, None, None, 0.0, table,
                                step.positions, held.pages, view.write_page, view.write_off, view.page_size,
-                               bias=self.bias)
-        out = attend(k, q, held, view, step, self.kv_heads, self.vdim, self.sink if self.has_sink else None, self.scale,
+                               bias=self.bias, values="keys" if self.values_from_keys else "own")
+        sink = self.sink if self.has_sink else self.fixed_sink
+        out = attend(k, q, held, view, step, self.kv_heads, self.vdim, sink, self.scale,
                      self.window, self.softcap, (self.r1, self.r2) if self.distance_bias else None, self.keep_first)
-        return self.o(out)
+        if self.has_gate:
+            k.head_gate(out, qkv[:, self.qkv_width: self.qkv_width + self.heads], self.heads)
+        out = self.o(out)
+        return k.add_bias(out, self.o_bias) if self.has_o_bias else out
 
     __call__ = forward
 
