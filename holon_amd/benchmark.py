@@ -24,7 +24,8 @@ prompts of 32,768 tokens at the Qwen3-4B shape, 512 tokens each at temperature 0
 --workload tolurax (or relanex, or nevodra) measures that design beside Qwen3 at equal sizes (width, layers, heads, head size,
 feed-forward, vocabulary; random weights): a 2,048-token prompt and decode at batch 8 near a context of 2,048, at two
 sizes (`--sizes`), one line with both models' figures and the bytes a decode step must read. `--only` runs one model
-(for a profiler).
+(for a profiler). --workload dopirax measures Dopirax the same way, beside Nevodra (the nearest design: both sublayers
+on one float32 stream, a capped attention, experts) and Qwen3 (`--beside`).
 """
 from __future__ import annotations
 
@@ -166,7 +167,33 @@ def nevodra_config(z: dict, window: int = 1024) -> dict:
             "embedding": {"scale": 1.0}, "canon": {"taps": 3}, "layers": [layer(i) for i in range(z["layers"])]}
 
 
-DESIGN_CONFIGS = {"tolurax": tolurax_config, "relanex": relanex_config, "nevodra": nevodra_config}
+def dopirax_config(z: dict) -> dict:
+    """A Dopirax model of a size's layers, in fours: differential attention with half the size's heads (two maps a
+    head, so as many score maps as the size has heads; keys and values of the size's head size, all of a map turned)
+    over a dense feed-forward of the size's width; a second such layer that reads the first one's keys and values, over
+    eight experts of a quarter of that width of which a token uses two, beside a gated shared one; then two layers of
+    the attention whose values are its keys (the size's heads, half of a head turned, a cap of 30, a gate a head), one
+    over the experts and one over the dense feed-forward."""
+    quarter = z["ff"] // 4
+    experts = {"kind": "moe", "expert": {"ff": quarter}, "shared": {"ff": quarter}, "router": {"experts": 8, "top": 2}}
+    dense = {"kind": "dense", "ff": z["ff"]}
+
+    def layer(i: int) -> dict:
+        if i % 4 < 2:
+            m = {"heads": z["heads"] // 2, "kv_heads": max(z["kv_heads"] // 2, 1), "dim": z["dim"], "vdim": z["dim"],
+                 "scale": z["dim"] ** -0.5, "diff": 0.5, "rot": {"dims": z["dim"], "base": 1e6}}
+            if i % 4 == 1:
+                m["kv_from"] = i - 1
+            return {"type": "attention_2", "mixer": m, "mlp": dense if i % 4 == 0 else experts}
+        m = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "scale": z["dim"] ** -0.5,
+             "softcap": 30.0, "rot": {"dims": z["dim"] // 2, "base": 1e6}}
+        return {"type": "attention", "mixer": m, "mlp": experts if i % 4 == 2 else dense}
+    return {"architecture": "Dopirax", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "layers": [layer(i) for i in range(z["layers"])]}
+
+
+DESIGN_CONFIGS = {"tolurax": tolurax_config, "relanex": relanex_config, "nevodra": nevodra_config,
+                  "dopirax": dopirax_config}
 
 
 def design_cache_bytes(name: str, cfg_json: dict, z: dict, item: int, batch: int, context: int) -> int:
@@ -176,7 +203,10 @@ def design_cache_bytes(name: str, cfg_json: dict, z: dict, item: int, batch: int
     total = 0
     for layer in cfg_json["layers"]:
         m = layer["mixer"]
-        if layer["type"] == "parallel":             # the window's keys and values
+        if name == "dopirax":                       # every layer reads all of a cache, its own or another layer's; the
+            maps = 2 if layer["type"] == "attention_2" else 1     # differential layers keep keys and values for each map
+            total += maps * m["kv_heads"] * (m["dim"] + m["vdim"]) * item * batch * context
+        elif layer["type"] == "parallel":             # the window's keys and values
             total += 2 * z["kv_heads"] * z["dim"] * item * batch * min(context, m["left"]["mask"]["size"])
         elif layer["type"] == "attention":
             seen = min(context, m["mask"]["size"] + m["mask"].get("keep_first", 0)) if m.get("mask") else context
@@ -209,7 +239,9 @@ def design(a) -> int:
     for size in a.sizes.split(","):
         z = DESIGN_SIZES[size]
         ours = DESIGN_CONFIGS[a.workload](z)
-        for name, cfg_json in ((a.workload, ours), ("qwen3", qwen3_config(z))):
+        others = [n for n in (a.beside or ("nevodra,qwen3" if a.workload == "dopirax" else "qwen3")).split(",") if n]
+        beside = [(n, qwen3_config(z) if n == "qwen3" else DESIGN_CONFIGS[n](z)) for n in others if n != a.workload]
+        for name, cfg_json in [(a.workload, ours)] + beside:
             if a.only and a.only != name:
                 continue
             engine = Engine.from_random(cfg_json, seed=0, cfg=EngineConfig(
@@ -258,7 +290,7 @@ def design(a) -> int:
             del engine
             gc.collect()
             torch.cuda.empty_cache()
-    print(json.dumps({"metric": f"{a.workload.capitalize()} beside Qwen3 at equal sizes: 2,048-token prompt, decode at batch 8 near "
+    print(json.dumps({"metric": f"{a.workload.capitalize()} beside {' and '.join(n.capitalize() for n in others)} at equal sizes: 2,048-token prompt, decode at batch 8 near "
                                 "context 2,048",
                       "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
                       "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
@@ -281,10 +313,14 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--context", type=int, default=CONTEXT, help="the context the timed decode steps end at")
     ap.add_argument("--prompt", type=int, default=PROMPT, help="tokens of the timed prompt")
     ap.add_argument("--no-graphs", action="store_true")
-    ap.add_argument("--workload", choices=("decode", "mixed", "long", "tolurax", "relanex", "nevodra"), default="decode")
-    ap.add_argument("--sizes", default="2k,4k", help="--workload tolurax|relanex|nevodra: which of its sizes (2k, 4k) to run")
-    ap.add_argument("--only", choices=("tolurax", "relanex", "nevodra", "qwen3"), default=None,
-                    help="--workload tolurax|relanex|nevodra: one model only")
+    ap.add_argument("--workload", choices=("decode", "mixed", "long", "tolurax", "relanex", "nevodra", "dopirax"),
+                    default="decode")
+    ap.add_argument("--sizes", default="2k,4k", help="--workload tolurax|relanex|nevodra|dopirax: which of its sizes (2k, 4k) to run")
+    ap.add_argument("--only", choices=("tolurax", "relanex", "nevodra", "dopirax", "qwen3"), default=None,
+                    help="--workload tolurax|relanex|nevodra|dopirax: one model only")
+    ap.add_argument("--beside", default=None,
+                    help="--workload of a design: the models it is measured beside, with commas (default: qwen3; for "
+                         "dopirax: nevodra,qwen3)")
     ap.add_argument("--products", choices=("own", "vendor", "timed"), default="timed",
                     help="EngineConfig.products: which kernel products of 17 to 1,024 rows take (reported in the line)")
     a = ap.parse_args(argv)

@@ -185,8 +185,8 @@ class RMSNorm32(NormPart):
     def add(self, x, residual: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         """(norm(residual + x), residual + x): `residual` is float32 and takes the sum in place; `x` is a tensor or
         `Pending` terms."""
-        return self.kernels.stream_rms(residual, _terms(x), None, self.weight, None, self.eps, self.build.dtype)[0], \
-            residual
+        return self.kernels.stream_rms(residual, _terms(x), getattr(x, "row", None), self.weight, None, self.eps,
+                                       self.build.dtype)[0], residual
 
     def fusion(self) -> dict | None:
         return {"norm": "rmsnorm", "eps": self.eps, "weight": self.weight}
@@ -246,6 +246,9 @@ class Parallel32(Part):
                 raise ValueError(f"pass {site.turn} of a range that has vectors for {self.passes} passes")
             row = self.step[site.turn]
         terms = _terms(stream.delta)
+        waiting = getattr(stream.delta, "row", None)       # a bias the layer before left to add to every row
+        if waiting is not None:
+            row = waiting if row is None else row + waiting
         stream.delta = stream.stats = None
         if self._fused_filter and step.rows.in_order:      # single tokens: the norms and both filters in one kernel
             second = self.conv2 is not None
@@ -253,7 +256,7 @@ class Parallel32(Part):
                                        self._one_kernel, self.build.dtype, self.conv1.weight,
                                        self.conv2.weight if second else None, site.slot_state[self.conv1.name],
                                        site.slot_state[self.conv2.name] if second else None, step.slots, step.starts)
-            stream.delta = Pending([(t, 1.0) for t in self._mix(a, b, step, site)])
+            stream.delta = self._pending(a, b, step, site)
             return stream
         if self._one_kernel is not None:
             a, b = k.stream_rms(h, terms, row, self.norm1.weight, self.norm2.weight if self.norm2 is not None else None,
@@ -267,14 +270,17 @@ class Parallel32(Part):
             a = self.conv1(a, step, site)
         if self.ffn is not None and self.conv2 is not None:
             b = self.conv2(b, step, site)
-        stream.delta = Pending([(t, 1.0) for t in self._mix(a, b, step, site)])
+        stream.delta = self._pending(a, b, step, site)
         return stream
 
-    def _mix(self, a, b, step, site) -> list[torch.Tensor]:
-        """Both sublayers' results from their inputs (one input for both under `shared_norm`)."""
-        out = [self.mixer(a, step, site)]
+    def _pending(self, a, b, step, site) -> Pending:
+        """Both sublayers' results from their inputs (one input for both under `shared_norm`), as terms for the next
+        norm's kernel. A mixer that names a bias on its last projection (`out_row`, a float32 vector) is asked to
+        leave it out (`add_row=False`): it joins the stream in float32, in the same kernel as the terms."""
+        row = getattr(self.mixer, "out_row", None)
+        out = [self.mixer(a, step, site) if row is None else self.mixer(a, step, site, add_row=False)]
         if self.ffn is not None:
             out.append(self.ffn(a if self.shared_norm else b, step))
-        return out
+        return Pending([(t, 1.0) for t in out], row)
 
     __call__ = forward

@@ -442,7 +442,12 @@ class SoftmaxAttention(Part):
     def extra_tensors(self):
         return [t for t in (self.bias, self.fixed_sink) if t is not None]
 
-    def forward(self, x: torch.Tensor, step, site) -> torch.Tensor:
+    @property
+    def out_row(self) -> torch.Tensor | None:
+        """The output projection's bias, for a caller that adds it to the stream itself (`forward(add_row=False)`)."""
+        return self.o_bias if self.has_o_bias else None
+
+    def forward(self, x: torch.Tensor, step, site, add_row: bool = True) -> torch.Tensor:
         k = self.kernels
         held = site.paged[self.state_name]
         view = step.paged[held.group]
@@ -462,7 +467,7 @@ class SoftmaxAttention(Part):
         if self.has_gate:
             k.head_gate(out, qkv[:, self.qkv_width: self.qkv_width + self.heads], self.heads)
         out = self.o(out)
-        return k.add_bias(out, self.o_bias) if self.has_o_bias else out
+        return k.add_bias(out, self.o_bias) if self.has_o_bias and add_row else out
 
     __call__ = forward
 

@@ -117,16 +117,17 @@ register_kernel(KernelOp("softcap", softcap_plain, "holon_softcap", [_P, _L, _F]
 
 # -- parts ------------------------------------------------------------------------------------------------------------
 class Pending:
-    """Terms not yet added to a float32 stream: [(tensor [T, W], scale)]. The next norm's kernel adds them as it
-    reads the rows."""
+    """Terms not yet added to a float32 stream: [(tensor [T, W], scale)], and optionally `row`, one float32 vector [W]
+    that is added to every row (a projection's bias that waits for the same add). The next norm's kernel adds them as
+    it reads the rows; a norm whose kernel takes no such vector is not handed one."""
 
-    def __init__(self, terms: list[tuple[torch.Tensor, float]]) -> None:
-        self.terms = terms
+    def __init__(self, terms: list[tuple[torch.Tensor, float]], row: torch.Tensor | None = None) -> None:
+        self.terms, self.row = terms, row
 
     def index_select(self, dim: int, index: torch.Tensor) -> "Pending":
         if dim != 0:
             raise ValueError("Pending.index_select: rows only (dim 0)")
-        return Pending([(t.index_select(0, index), s) for t, s in self.terms])
+        return Pending([(t.index_select(0, index), s) for t, s in self.terms], self.row)
 
 
 def _terms(x) -> list[tuple[torch.Tensor, float]]:
