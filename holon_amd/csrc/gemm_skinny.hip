@@ -191,6 +191,12 @@ __global__ void __launch_bounds__(WPB * 64) gemm_skinny_kernel(const bf16_t* __r
         ushort4 o;
         o.x = float_to_bf16(acc[j][0]); o.y = float_to_bf16(acc[j][1]);
         o.z = float_to_bf16(acc[j][2]); o.w = float_to_bf16(acc[j][3]);
+        if (round_first == 4) {      // the squared ReLU of the rounded product, rounded: the two kernels' roundings in one
+          const float v0 = fmaxf(bf16_to_float(o.x), 0.f), v1 = fmaxf(bf16_to_float(o.y), 0.f);
+          const float v2 = fmaxf(bf16_to_float(o.z), 0.f), v3 = fmaxf(bf16_to_float(o.w), 0.f);
+          o.x = float_to_bf16(v0 * v0); o.y = float_to_bf16(v1 * v1);
+          o.z = float_to_bf16(v2 * v2); o.w = float_to_bf16(v3 * v3);
+        }
         if constexpr (RESID) {
           const ushort4 r = before[j];
           o.x = float_to_bf16(bf16_to_float(r.x) + bf16_to_float(o.x));
@@ -262,13 +268,16 @@ extern "C" int holon_gemm_skinny_supported(int M, int N, int K) {
 }
 
 // out_f32: 0 writes bfloat16, 1 float32 straight from the accumulators, 2 float32 values that were rounded to bfloat16
-// first (the product in the operands' type, cast up). tiled: 1 when `w` is in the tile layout (see holon_tile_weight_bf16).
+// first (the product in the operands' type, cast up), 4 bfloat16 again: max(product, 0)^2 of the rounded product (a
+// feed-forward's squared ReLU in the product's epilogue). tiled: 1 when `w` is in the tile layout (see holon_tile_weight_bf16).
 extern "C" int holon_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_f32,
                                       int tiled, void* stream) {
   HOLON_CHECK(holon_gemm_skinny_supported(M, N, K), "gemm (few rows): M=%d N=%d K=%d not served (M <= 16, N %% 16, K %% 32)",
               M, N, K);
   hipStream_t s = (hipStream_t)stream;
-  if (out_f32) pick_waves<float>(x, w, y, M, N, K, tiled != 0, s, out_f32 == 2);
+  HOLON_CHECK(out_f32 == 0 || out_f32 == 1 || out_f32 == 2 || out_f32 == 4, "gemm (few rows): no output form %d", out_f32);
+  if (out_f32 == 4) pick_waves<bf16_t>(x, w, y, M, N, K, tiled != 0, s, 4);
+  else if (out_f32) pick_waves<float>(x, w, y, M, N, K, tiled != 0, s, out_f32 == 2);
   else pick_waves<bf16_t>(x, w, y, M, N, K, tiled != 0, s);
   HOLON_LAUNCH_OK();
   return 0;

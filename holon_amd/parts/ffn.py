@@ -219,6 +219,30 @@ register_kernel(KernelOp("moe_router_top", moe_router_top_plain, "holon_moe_rout
 register_kernel(KernelOp("relu2", relu2_plain, "holon_relu2", [_P, _P, _L, _I], _relu2_hip))
 
 
+def linear_relu2_plain(x, weight, tiled=None):
+    """relu2(x W^T) where one kernel does both, with the roundings of the two one after the other; None where it does
+    not (the caller then composes them). The plain form never does."""
+    return None
+
+
+def _linear_relu2_hip(launch, x, weight, tiled=None):
+    """Steps of up to 16 bfloat16 rows: the few-row product with the activation in its epilogue."""
+    (m, k), n = x.shape, weight.shape[0]
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.is_contiguous()
+            and weight.is_contiguous() and weight.shape[1] == k and 1 <= m <= 16 and n % 16 == 0 and k % 32 == 0
+            and k >= 256 and (tiled is None or (tiled.shape == weight.shape and tiled.dtype == weight.dtype
+                                                 and tiled.is_contiguous()))):
+        return None
+    y = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    launch(x.data_ptr(), (tiled if tiled is not None else weight).data_ptr(), y.data_ptr(), m, n, k, 4,
+           int(tiled is not None))
+    return y
+
+
+register_kernel(KernelOp("linear_relu2", linear_relu2_plain, "holon_gemm_skinny_bf16", [_P, _P, _P, _I, _I, _I, _I, _I],
+                         _linear_relu2_hip))
+
+
 @register_part("ffn", "polynorm")
 class PolyNormFFN(Part):
     """down(act(up(x))) with act = a N(z) + b N(z^2) + c N(z^3) + e (`act` holds a, b, c, e; N divides a token's
@@ -255,7 +279,11 @@ class DenseFFN(Part):
         self.attach("down_proj", Linear(build, inp=inter, out=hidden))
 
     def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
-        return self.down_proj(self.kernels.relu2(self.up_proj(x)))
+        up = self.up_proj
+        y = self.kernels.linear_relu2(x, up.weight, up.tiled if up.folded is None else None)
+        if y is None:
+            y = self.kernels.relu2(up(x))
+        return self.down_proj(y)
 
     __call__ = forward
 

@@ -494,6 +494,14 @@ def test_kernels_alone_against_their_plain_forms(dtype):
     for n in (5, 77 * 3, 4096 * 9):
         z = randn(n // 1 if n < 100 else n // 3, 1 if n < 100 else 3)
         assert H.rel_rms(k.relu2(z), kernel_op("relu2").plain(z)) < tol
+    if dtype == torch.bfloat16:                    # the activation in the few-row product's epilogue
+        for m, n, kk in ((1, 64, 256), (8, 320, 512), (16, 2048, 1024), (5, 48, 288)):
+            x, w = randn(m, kk), randn(n, kk) * kk ** -0.5
+            tiled = k.tile_weight(w)
+            for copy in (None, tiled):
+                fused = k.linear_relu2(x, w, copy)
+                assert fused is not None and H.rel_rms(fused, k.relu2(k.linear(x, w, None, copy))) < 1e-6, (m, n, kk)
+        assert k.linear_relu2(randn(17, 256), randn(64, 256), None) is None
     for heads, vdim, extra in ((4, 24, 16), (3, 64, 5), (16, 128, 0)):
         x, wide = randn(9, heads * vdim), randn(9, 40 + heads + extra)
         gates = wide[:, 40: 40 + heads]
@@ -565,3 +573,67 @@ def test_kernels_alone_against_their_plain_forms(dtype):
         qc = prepare(only_q, heads, 0, dim, vdim, qw, kw, 1e-6, tab, positions, None, None, None, page,
                      bias=None if bias is None else bias[: heads * dim].contiguous())
         assert H.rel_rms(qa, qc) < tol and torch.equal(qc, qb), "queries alone"
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_a_shared_prefix_through_the_engine(folders, device):
+    """Every layer's state lies in pages without a window, so a request may start from the pages of an earlier one
+    with the same first tokens, the layers that read another layer's cache included: the second request skips the
+    shared pages and still generates what the plain model generates."""
+    from holon_amd.config import EngineConfig, SamplingParams
+    from holon_amd.engine.engine import Engine
+    folder = folders["A-sharp"]
+    plain_model = _plain(str(folder))
+    head = H.random_ids(43, M.CONFIG_A["vocab"], 7)
+    prompts = [head + H.random_ids(5, M.CONFIG_A["vocab"], 8), head + H.random_ids(9, M.CONFIG_A["vocab"], 9)]
+    engine = Engine(EngineConfig(model=str(folder), device=device, dtype="float32", page_size=8, max_seqs=2,
+                                 max_model_len=96, max_step_tokens=64, cache_tokens=192),
+                    TorchKernels() if device == "cpu" else None)
+    params = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
+    outs = [engine.generate([p], params)[0] for p in prompts]
+    assert engine.stats()["prefix_tokens_saved"] >= 40
+    held = sum(H.assert_greedy_follows(plain_model, p, o, margin=0.02) for p, o in zip(prompts, outs))
+    assert held >= 18
+    engine.cache.check()
+    engine.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dim", [64, 128, 256])
+def test_the_cap_and_the_fixed_sink_on_the_matrix_cores(dim):
+    """`paged_attention` as the attention mixer calls it (all keys before the query, a cap or none, a sink of 0 for
+    every head), in bfloat16 at every head size the matrix cores serve, prompt portions beside decode rows over
+    scattered pages, short rows among them (where the one in the denominator weighs most), against float64."""
+    from holon_amd.kernels import load_hip
+    from holon_amd.kernels.api import AttnRows
+    k, dev, page, heads, groups = load_hip(), "cuda", 16, 8, 2
+    g = torch.Generator().manual_seed(dim + 1)
+    lens, counts = [300, 75, 190, 3, 129, 1, 40], [300, 1, 60, 3, 1, 1, 2]     # tokens a row holds, and brings in this step
+    n_pages = sum(-(-n // page) for n in lens) + 1
+    table = torch.full((len(lens) + 1, 24), n_pages - 1, dtype=torch.int32)
+    order, at = torch.randperm(n_pages - 1, generator=g).tolist(), 0
+    for s_, n in enumerate(lens):
+        for i in range(-(-n // page)):
+            table[s_, i] = order[at]
+            at += 1
+    pages = (torch.randn(n_pages, 2, groups, page * dim, generator=g) * 0.5).to(dev).bfloat16()
+    qstart = [0]
+    for c in counts:
+        qstart.append(qstart[-1] + c)
+    q = torch.randn(qstart[-1], heads, dim, generator=g).to(dev).bfloat16()
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)          # noqa: E731
+    decode = [b for b, c in enumerate(counts) if c == 1]
+    chunk = [b for b, c in enumerate(counts) if c > 1]
+    rows = AttnRows(slots=i32(list(range(len(lens)))), lens=i32(lens), query_start=i32(qstart), decode_rows=i32(decode),
+                    chunk_rows=i32(chunk), n_decode=len(decode), n_chunk=len(chunk),
+                    max_decode_len=max(lens[b] for b in decode), max_chunk_query=max(counts),
+                    max_chunk_len=max(lens[b] for b in chunk))
+    sink = torch.zeros(heads, device=dev)
+    twin = TorchKernels()
+    for scale, cap in ((2.0 * dim ** -0.5, 3.0), (dim ** -0.5, 30.0), (dim ** -0.5, 0.0), (0.05 * dim ** -0.5, 0.0)):
+        got = k.paged_attention(q, pages, table.to(dev), rows, page, scale, 0, sink=sink, softcap=cap)
+        want = twin.paged_attention(q.double(), pages.double(), table.to(dev), rows, page, scale, 0, sink=sink.double(),
+                                    softcap=cap)
+        assert H.rel_rms(got, want) < 8e-3, (dim, scale, cap)
+        per = ((got.double() - want).square().mean((1, 2)).sqrt() / want.square().mean().sqrt()).max().item()
+        assert per < 4e-2, (dim, scale, cap, per)
