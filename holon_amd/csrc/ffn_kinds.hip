@@ -218,38 +218,78 @@ __global__ void __launch_bounds__(256) moe_gate_kernel(const T* __restrict__ gat
     }
   }
 }
-// The other router, one block of 256 threads a token: float32 logits z_e = x . router[e] + bias[e] as above; the `top`
-// largest are chosen (equal ones: the lower index first) and weighted by the softmax over the chosen logits alone, every
-// other expert 0. Rows of `router` beyond the experts are gates: their columns hold sigmoid(x . router[r]).
+// The other router, one block of 256 threads a token: float32 logits z_e = x . router[e] + bias[e]; the `top` largest
+// are chosen (equal ones: the lower index first) and weighted by the softmax over the chosen logits alone, every other
+// expert 0. Rows of `router` beyond the experts are gates: their columns hold sigmoid(x . router[r]).
+// Every thread takes a slice of the token's row against all router rows, sixteen rows at a time (their loads do not
+// wait for each other); a wave's lanes are summed by shuffles and the four waves' partial sums in wave order. Up to 64
+// experts one wave then makes the choice with an expert a lane; more are ranked by the whole block.
 template <typename T>
 __global__ void __launch_bounds__(256) moe_router_top_kernel(const T* __restrict__ x, const float* __restrict__ router,
                                                              const float* __restrict__ bias, float* __restrict__ weights,
                                                              int width, int experts, int rows_r, int top) {
-  extern __shared__ float xs[];                          // [width]
+  __shared__ float part_s[4][ROUTE_MAX_E + 1];
   __shared__ float z_s[ROUTE_MAX_E + 1];
   __shared__ float e_s[ROUTE_MAX_E];
   __shared__ float red_s[4];
   const int64_t t = blockIdx.x;
-  for (int i = threadIdx.x; i < width; i += 256) xs[i] = Elem<T>::load(x[t * width + i]);
-  __syncthreads();
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  const bool wide = width % 4 == 0 && (uintptr_t)router % 16 == 0;
-  for (int e = wave; e < rows_r; e += 4) {
-    const float* w = router + (int64_t)e * width;
-    float acc = 0.f;
+  const T* row = x + t * width;
+  const bool wide = width % 4 == 0 && (uintptr_t)router % 16 == 0 && (uintptr_t)x % 16 == 0;
+  for (int e0 = 0; e0 < rows_r; e0 += 16) {
+    float acc[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[j] = 0.f;
     if (wide) {
-      for (int i = lane * 4; i < width; i += WAVE * 4) {
-        const float4 v = *reinterpret_cast<const float4*>(w + i);
-        acc += xs[i] * v.x + xs[i + 1] * v.y + xs[i + 2] * v.z + xs[i + 3] * v.w;
+      for (int i = threadIdx.x * 4; i < width; i += 1024) {
+        const float x0 = Elem<T>::load(row[i]), x1 = Elem<T>::load(row[i + 1]), x2 = Elem<T>::load(row[i + 2]),
+                    x3 = Elem<T>::load(row[i + 3]);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          if (e0 + j < rows_r) {
+            const float4 v = *reinterpret_cast<const float4*>(router + (int64_t)(e0 + j) * width + i);
+            acc[j] += x0 * v.x + x1 * v.y + x2 * v.z + x3 * v.w;
+          }
+        }
       }
     } else {
-      for (int i = lane; i < width; i += WAVE) acc += xs[i] * w[i];
+      for (int i = threadIdx.x; i < width; i += 256) {
+        const float xv = Elem<T>::load(row[i]);
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+          if (e0 + j < rows_r) acc[j] += xv * router[(int64_t)(e0 + j) * width + i];
+      }
     }
-    acc = wave_sum(acc);
-    if (lane == 0) z_s[e] = e < experts ? acc + (bias ? bias[e] : 0.f) : acc;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      if (e0 + j < rows_r) {
+        const float a = wave_sum(acc[j]);
+        if (lane == 0) part_s[wave][e0 + j] = a;
+      }
+    }
   }
   __syncthreads();
-  // the largest logit is always chosen: the softmax over the chosen ones is taken about it
+  auto logit = [&](int e) {
+    const float z = ((part_s[0][e] + part_s[1][e]) + part_s[2][e]) + part_s[3][e];
+    return e < experts && bias ? z + bias[e] : z;
+  };
+  if (experts <= WAVE) {                                  // an expert a lane
+    if (wave != 0) return;
+    const float mine = lane < experts ? logit(lane) : -INFINITY;
+    int ahead = 0;
+    for (int o = 0; o < experts; ++o) {
+      const float other = __shfl(mine, o, WAVE);
+      ahead += (other > mine) || (other == mine && o < lane);
+    }
+    const float top_z = wave_max(mine);                   // the largest logit is always chosen
+    const float v = lane < experts && ahead < top ? expf(mine - top_z) : 0.f;
+    const float sum = wave_sum(v);
+    if (lane < experts) weights[t * rows_r + lane] = v / sum;
+    if (rows_r > experts && lane == 0) weights[t * rows_r + experts] = 1.0f / (1.0f + expf(-logit(experts)));
+    return;
+  }
+  for (int e = threadIdx.x; e < rows_r; e += 256) z_s[e] = logit(e);
+  __syncthreads();
   float top_z = -INFINITY;
   for (int e = threadIdx.x; e < experts; e += 256) top_z = fmaxf(top_z, z_s[e]);
   top_z = wave_max(top_z);
@@ -393,13 +433,12 @@ extern "C" int holon_moe_router_top(const void* x, const float* router, const fl
               (long long)rows, width, top, experts, ROUTE_MAX_E, router_rows);
   if (rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  const size_t lds = (size_t)width * sizeof(float);
   if (dtype == HOLON_F32)
-    moe_router_top_kernel<float><<<(unsigned)rows, 256, lds, s>>>((const float*)x, router, bias, weights, width,
-                                                                 experts, router_rows, top);
+    moe_router_top_kernel<float><<<(unsigned)rows, 256, 0, s>>>((const float*)x, router, bias, weights, width, experts,
+                                                               router_rows, top);
   else
-    moe_router_top_kernel<bf16_t><<<(unsigned)rows, 256, lds, s>>>((const bf16_t*)x, router, bias, weights, width,
-                                                                  experts, router_rows, top);
+    moe_router_top_kernel<bf16_t><<<(unsigned)rows, 256, 0, s>>>((const bf16_t*)x, router, bias, weights, width,
+                                                                experts, router_rows, top);
   HOLON_LAUNCH_OK();
   return 0;
 }

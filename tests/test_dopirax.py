@@ -333,7 +333,7 @@ def test_the_router_chooses_as_the_plain_model(device):
         router_top = kernel_op("moe_router_top").plain
     g = torch.Generator().manual_seed(3)
     for experts, top, width, gated in ((8, 3, 64, True), (12, 4, 250, False), (6, 6, 32, True), (16, 1, 100, True), (1, 1, 8, True),
-                                       (64, 6, 512, False)):
+                                       (64, 6, 512, False), (130, 9, 48, True)):
         x = torch.randn(50, width, generator=g).to(device)
         router = (2.0 * torch.randn(experts + int(gated), width, generator=g) * width ** -0.5).to(device)
         router[1] = router[0]                      # two experts with equal logits (their biases are made equal below)
@@ -527,7 +527,8 @@ def test_kernels_alone_against_their_plain_forms(dtype):
         assert H.rel_rms(a, kernel_op("moe_gate").plain(gate_up, weights, ff, shared, shared_weight=True)) < tol
         a = k.moe_gate(gate_up, weights[:, :experts].contiguous(), ff, shared)
         assert H.rel_rms(a, kernel_op("moe_gate").plain(gate_up, weights[:, :experts].contiguous(), ff, shared)) < tol
-    for experts, top, width, rows in ((8, 3, 256, 9), (12, 4, 250, 12), (64, 6, 2048, 65), (5, 1, 77, 5), (1, 1, 16, 2)):
+    for experts, top, width, rows in ((8, 3, 256, 9), (12, 4, 250, 12), (64, 6, 2048, 65), (5, 1, 77, 5), (1, 1, 16, 2),
+                                      (100, 7, 320, 101), (300, 2, 96, 300), (17, 17, 1024, 18)):
         x, router = randn(19, width), randn(rows, width, to=torch.float32) * 0.2
         bias = randn(experts, to=torch.float32) * 0.5
         got = k.moe_router_top(x, router, bias, experts, top)
