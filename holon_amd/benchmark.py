@@ -203,9 +203,9 @@ def design_cache_bytes(name: str, cfg_json: dict, z: dict, item: int, batch: int
     total = 0
     for layer in cfg_json["layers"]:
         m = layer["mixer"]
-        if name == "dopirax":                       # every layer reads all of a cache, its own or another layer's; the
-            maps = 2 if layer["type"] == "attention_2" else 1     # differential layers keep keys and values for each map
-            total += maps * m["kv_heads"] * (m["dim"] + m["vdim"]) * item * batch * context
+        if name == "dopirax":                       # every layer reads all of a cache, its own or another layer's
+            maps = 2 if layer["type"] == "attention_2" else 1     # differential layers keep the keys of both maps
+            total += m["kv_heads"] * (maps * m["dim"] + m["vdim"]) * item * batch * context
         elif layer["type"] == "parallel":             # the window's keys and values
             total += 2 * z["kv_heads"] * z["dim"] * item * batch * min(context, m["left"]["mask"]["size"])
         elif layer["type"] == "attention":

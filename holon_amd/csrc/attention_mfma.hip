@@ -72,7 +72,18 @@ struct AttnArgs {
   const float* r1;
   const float* r2;
   int keep_first;
+  // key heads that share one value head (0 or 1: every key head has its own): a page then holds kv_heads planes of
+  // keys and kv_heads / v_share planes of values, and key head hk reads value head hk / v_share
+  int v_share;
 };
+
+// The planes (one head's P tokens of keys or of values) a page holds, and the plane of key head hk's values.
+__device__ __forceinline__ int64_t page_planes(const AttnArgs& a) {
+  return a.v_share > 1 ? a.kv_heads + a.kv_heads / a.v_share : 2 * (int64_t)a.kv_heads;
+}
+__device__ __forceinline__ int64_t value_plane(const AttnArgs& a, int hk) {
+  return (int64_t)a.kv_heads + (a.v_share > 1 ? hk / a.v_share : hk);
+}
 
 // What a lane needs to change its column's scores: the head's two numbers of the distance bias.
 struct ModLane {
@@ -210,9 +221,9 @@ __device__ __forceinline__ void attn_tiles(const AttnArgs& a, const int32_t* __r
   const int g = lane / 16, c = lane % 16;
   const int P = a.page_size;
   const int64_t plane = (int64_t)P * D;
-  const int64_t page_stride = 2 * (int64_t)a.kv_heads * plane;
+  const int64_t page_stride = page_planes(a) * plane;
   const bf16_t* kbase = a.pages + (int64_t)hk * plane;
-  const bf16_t* vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
+  const bf16_t* vbase = a.pages + value_plane(a, hk) * plane;
   const int krow = 8 * (c / 4) + (c % 4);   // this lane's key (row of A) within the 32-key block, first product
   const int khalf = krow / 16, kin = krow % 16;
   const int max_page = a.table_stride - 1;
@@ -470,9 +481,9 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
   const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
   const int P = a.page_size;
   const int64_t plane = (int64_t)P * D;
-  const int64_t page_stride = 2 * (int64_t)a.kv_heads * plane;
+  const int64_t page_stride = page_planes(a) * plane;
   const bf16_t* kbase = a.pages + (int64_t)hk * plane;
-  const bf16_t* vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
+  const bf16_t* vbase = a.pages + value_plane(a, hk) * plane;
   const int max_page = min(a.table_stride, PG) - 1;
 
   // every entry a stage can ask for: the last stage's second half may lie one page past the row's tokens (the table
@@ -691,9 +702,9 @@ __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kerne
   const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
   const int P = a.page_size;
   const int64_t plane = (int64_t)P * D;
-  const int64_t page_stride = 2 * (int64_t)a.kv_heads * plane;
+  const int64_t page_stride = page_planes(a) * plane;
   const bf16_t* kbase = a.pages + (int64_t)hk * plane;
-  const bf16_t* vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
+  const bf16_t* vbase = a.pages + value_plane(a, hk) * plane;
   const int max_page = min(a.table_stride, PG) - 1;
   for (int i = tid; i < min(PG, a.table_stride); i += 256) pg_lds[i] = trow[i];
   constexpr int KCH = D / 8;
@@ -1004,9 +1015,9 @@ struct StagedCopies {
     pg = pg_lds;
     P = a.page_size;
     const int64_t plane = (int64_t)P * D;
-    page_stride = 2 * (int64_t)a.kv_heads * plane;
+    page_stride = page_planes(a) * plane;
     kbase = a.pages + (int64_t)hk * plane;
-    vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
+    vbase = a.pages + value_plane(a, hk) * plane;
     max_page = min(a.table_stride, PG) - 1;
     const int lane = threadIdx.x % WAVE, h = lane / 32, c = lane % 32;
     wave = threadIdx.x / WAVE;
@@ -1235,9 +1246,9 @@ __global__ void __launch_bounds__(256, 1) attn_prefill_pair_kernel(AttnArgs a) {
   const int32_t* trow = a.table + (int64_t)a.slots[b] * a.table_stride;
   const int P = a.page_size;
   const int64_t plane = (int64_t)P * D;
-  const int64_t page_stride = 2 * (int64_t)a.kv_heads * plane;
+  const int64_t page_stride = page_planes(a) * plane;
   const bf16_t* kbase = a.pages + (int64_t)hk * plane;
-  const bf16_t* vbase = a.pages + ((int64_t)a.kv_heads + hk) * plane;
+  const bf16_t* vbase = a.pages + value_plane(a, hk) * plane;
   const int max_page = min(a.table_stride, PG) - 1;
   for (int i = tid; i < min(PG, a.table_stride); i += 256) pg_lds[i] = trow[i];
   constexpr int KCH = D / 8;
@@ -1870,13 +1881,17 @@ struct ScoreMod {
 static int prefill_launch(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
                           const int32_t* slots, const int32_t* lens, const int32_t* query_start, const int32_t* row_ids,
                           int n_rows, int max_query, int max_len, int heads, int kv_heads, int head_dim, int page_size,
-                          float scale, int window, const float* sink, void* stream, const ScoreMod* mod = nullptr) {
+                          float scale, int window, const float* sink, void* stream, const ScoreMod* mod = nullptr,
+                          int v_share = 1) {
   HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
               "attention: bad sizes");
+  HOLON_CHECK(v_share >= 1 && kv_heads % v_share == 0, "attention: %d key heads do not share value heads by %d", kv_heads,
+              v_share);
   if (n_rows <= 0 || max_query <= 0) return 0;
   AttnArgs a{};
+  a.v_share = v_share;
   a.q = (const bf16_t*)q; a.out = (bf16_t*)out; a.pages = (const bf16_t*)pages; a.table = table;
   a.table_stride = table_stride; a.slots = slots; a.lens = lens; a.qstart = query_start; a.row_ids = row_ids;
   a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size;
@@ -2039,11 +2054,13 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
                          int n_rows, int max_len, int heads, int kv_heads, int head_dim, int page_size, float scale,
                          int window, float* part_o, float* part_ml, int splits, int keys_per_split, void* stream,
                          const FusedArgs* fused = nullptr, int waves = 1, int rows_in_order = 0,
-                         const float* sink = nullptr, const ScoreMod* mod = nullptr) {
+                         const float* sink = nullptr, const ScoreMod* mod = nullptr, int v_share = 1) {
   HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
               "attention: bad sizes");
+  HOLON_CHECK(v_share >= 1 && kv_heads % v_share == 0 && (v_share == 1 || fused == nullptr),
+              "attention: %d key heads do not share value heads by %d", kv_heads, v_share);
   HOLON_CHECK(splits > 0 && splits <= 64 && keys_per_split > 0 && keys_per_split % 32 == 0,
               "attention decode: %d splits of %d keys (1 to 64 splits of a multiple of 32 keys)", splits, keys_per_split);
   HOLON_CHECK(waves >= 1 && waves <= 8 && splits % waves == 0 && (waves - 1) * (16 * head_dim + 32) * 4 <= 64 * 1024,
@@ -2062,7 +2079,7 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
   a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size;
   a.scale_log2 = scale * 1.4426950408889634f; a.window = window;
   a.part_o = part_o; a.part_ml = part_ml; a.splits = splits; a.keys_per_split = keys_per_split;
-  a.out_splits = splits / waves; a.rows_in_order = rows_in_order; a.sink = sink;
+  a.out_splits = splits / waves; a.rows_in_order = rows_in_order; a.sink = sink; a.v_share = v_share;
   const TileMap tm = tile_map(heads / kv_heads);
   dim3 grid(a.out_splits, kv_heads * tm.head_blocks, n_rows);
   hipStream_t s = (hipStream_t)stream;
@@ -2165,6 +2182,38 @@ extern "C" int holon_attention_prefill_mod_bf16(const void* q, void* out, const 
   const ScoreMod mod{softcap, r1, r2, keep_first};
   return prefill_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_query, max_len,
                         heads, kv_heads, head_dim, page_size, scale, window, sink, stream, &mod);
+}
+
+// Prompt portions and decode rows over pages whose key heads share value heads: a page holds kv_heads planes of keys,
+// then kv_heads / v_share planes of values, and key head hk reads value head hk / v_share (several score maps over one
+// set of values). With a sink (nullable) and changed scores (softcap 0, r1 and r2 null, keep_first 0: none).
+extern "C" int holon_attention_prefill_shared_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                                   int table_stride, const int32_t* slots, const int32_t* lens,
+                                                   const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                                   int max_query, int max_len, int heads, int kv_heads, int head_dim,
+                                                   int page_size, float scale, int window, const float* sink,
+                                                   float softcap, const float* r1, const float* r2, int keep_first,
+                                                   int v_share, void* stream) {
+  const ScoreMod mod{softcap, r1, r2, keep_first};
+  const bool changed = softcap > 0.f || r1 != nullptr || (window > 0 && keep_first > 0);
+  return prefill_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_query, max_len,
+                        heads, kv_heads, head_dim, page_size, scale, window, sink, stream, changed ? &mod : nullptr,
+                        v_share);
+}
+
+extern "C" int holon_attention_decode_shared_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                                  int table_stride, const int32_t* slots, const int32_t* lens,
+                                                  const int32_t* query_start, const int32_t* row_ids, int n_rows,
+                                                  int max_len, int heads, int kv_heads, int head_dim, int page_size,
+                                                  float scale, int window, float* part_o, float* part_ml, int splits,
+                                                  int keys_per_split, int waves, int rows_in_order, const float* sink,
+                                                  float softcap, const float* r1, const float* r2, int keep_first,
+                                                  int v_share, void* stream) {
+  const ScoreMod mod{softcap, r1, r2, keep_first};
+  const bool changed = softcap > 0.f || r1 != nullptr || (window > 0 && keep_first > 0);
+  return decode_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len, heads,
+                       kv_heads, head_dim, page_size, scale, window, part_o, part_ml, splits, keys_per_split, stream,
+                       nullptr, waves, rows_in_order, sink, changed ? &mod : nullptr, v_share);
 }
 
 // Decode rows straight from the step's raw q/k/v projection: per-head norm, rotation and the cache write of each

@@ -82,6 +82,21 @@ int holon_attention_decode_sink_bf16(const void* q, void* out, const void* pages
                                      int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
                                      float* part_o, float* part_ml, int splits, int keys_per_split, int waves,
                                      int rows_in_order, const float* sink, void* stream);
+// Both over pages whose key heads share value heads: kv_heads planes of keys, then kv_heads / v_share planes of values
+// a page; key head hk reads value head hk / v_share. Sink nullable; softcap 0, r1 = r2 = null, keep_first 0: plain scores.
+int holon_attention_prefill_shared_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                        int table_stride, const int32_t* slots, const int32_t* lens,
+                                        const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_query,
+                                        int max_len, int heads, int kv_heads, int head_dim, int page_size, float scale,
+                                        int window, const float* sink, float softcap, const float* r1, const float* r2,
+                                        int keep_first, int v_share, void* stream);
+int holon_attention_decode_shared_bf16(const void* q, void* out, const void* pages, const int32_t* table,
+                                       int table_stride, const int32_t* slots, const int32_t* lens,
+                                       const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
+                                       int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
+                                       float* part_o, float* part_ml, int splits, int keys_per_split, int waves,
+                                       int rows_in_order, const float* sink, float softcap, const float* r1,
+                                       const float* r2, int keep_first, int v_share, void* stream);
 // The same from the step's raw q/k/v projection `qkv` [T, (heads + 2 kv_heads) head_dim]: per-head RMSNorm (q_weight
 // and k_weight, both or neither), rotation (rope_table [max_positions, head_dim] = cos | sin, or NULL) and the cache
 // write of every row's new token (write_page, write_off by token; its position is the row's len - 1) happen inside
@@ -241,7 +256,7 @@ int holon_head_prepare(const void* qkv, void* q_out, int tokens, int heads, int 
                        const void* q_weight, const void* k_weight, float eps, const float* table, int rot, int table_rows,
                        const int32_t* positions, void* pages, const int32_t* write_page, const int32_t* write_off,
                        int page_size, int num_pages, int dtype, const float* bias, int stride, int v_from_keys,
-                       int v_repeat, void* stream);
+                       int v_share, void* stream);
 int holon_sigmoid_attention(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
                             const int32_t* slots, const int32_t* token_row, const int32_t* positions,
                             const int32_t* query_start, const int32_t* row_ids, int tokens, int heads, int kv_heads,
@@ -271,12 +286,13 @@ int holon_dyt_stream(void* x, int x_dtype, const void* term, int term_dtype, con
 // (softmax_attention.hip) q [T, H, D] -> out [T, H V]; token t reads block table row slots[token_row[t]] and stands at
 // positions[t]; sink [H] float32 or null; window 0: everything before. softcap > 0: scores become softcap tanh(s /
 // softcap); r1, r2 [H] float32 (both or neither): r1 ln(1 + r2 (i - j)) is taken off the score of key j for query i;
-// keep_first: under a window, keys 0 .. keep_first - 1 stay visible.
+// keep_first: under a window, keys 0 .. keep_first - 1 stay visible. v_share > 1: a page holds kv_heads / v_share value
+// heads behind its kv_heads key heads, and key head h reads value head h / v_share.
 int holon_softmax_attention(const void* q, void* out, const void* pages, const int32_t* table, int table_stride,
                             int table_rows, const int32_t* slots, const int32_t* token_row, const int32_t* positions,
                             int tokens, int heads, int kv_heads, int dim, int vdim, int page_size, int num_pages,
                             const float* sink, float scale, int window, int dtype, float softcap, const float* r1,
-                            const float* r2, int keep_first, void* stream);
+                            const float* r2, int keep_first, int v_share, void* stream);
 // x [T, H V] *= sigmoid(gates[t, h]) per head (gates: columns of rows gate_stride apart); x [rows, dim] += bias;
 // y [T, 2 H V] (kv head, map, head in group) -> out [T, H V]: u = y1 - lam y2, u / sqrt(mean(u^2) + eps) * gain.
 int holon_head_gate(void* x, const void* gates, int64_t gate_stride, int64_t tokens, int heads, int vdim, int dtype,

@@ -17,9 +17,9 @@ namespace {
 
 // One wave per (token, head of q, k or v). A row of `qkv` is `stride` values long and holds q, k and v in its first
 // columns. `bias` (one float32 a column of q, k and v, or null) is added first. q and k: x * rsqrt(mean(x^2) + eps) *
-// weight (if weights), then the half-split rotation of the first `rot` dimensions; one rounding. Value head g of the
-// cache is projected value head g / v_repeat (several key heads over one value head), or, with `v_from_keys`, key head
-// g as projected (bias added, before norm and rotation; there are no value columns then). `pages` null: kv_heads is 0,
+// weight (if weights), then the half-split rotation of the first `rot` dimensions; one rounding. With `v_share`
+// s > 1 the row and the page hold kv_heads / s value heads (s key heads read one value head); with `v_from_keys` value
+// head g is key head g as projected (bias added, before norm and rotation; there are no value columns then). `pages` null: kv_heads is 0,
 // the rows hold queries alone and nothing is stored.
 template <typename T>
 __global__ void __launch_bounds__(256) head_prepare_kernel(const T* __restrict__ qkv, T* __restrict__ q_out, int heads,
@@ -30,20 +30,20 @@ __global__ void __launch_bounds__(256) head_prepare_kernel(const T* __restrict__
                                                            T* __restrict__ pages, const int32_t* __restrict__ write_page,
                                                            const int32_t* __restrict__ write_off, int page_size,
                                                            int num_pages, const float* __restrict__ bias, int64_t stride,
-                                                           int v_from_keys, int v_repeat) {
+                                                           int v_from_keys, int v_share) {
   const int t = blockIdx.x;
   const int hs = blockIdx.y * 4 + threadIdx.x / WAVE;
   const int lane = threadIdx.x % WAVE;
-  if (hs >= heads + 2 * kv_heads) return;
-  const int64_t page_len = (int64_t)kv_heads * page_size * (dim + vdim);
+  const int v_heads = kv_heads / v_share;
+  if (hs >= heads + kv_heads + v_heads) return;
+  const int64_t page_len = (int64_t)kv_heads * page_size * dim + (int64_t)v_heads * page_size * vdim;
   const T* row = qkv + (int64_t)t * stride;
   const int page = pages ? write_page[t] : -1, off = pages ? write_off[t] : -1;
   const bool page_ok = page >= 0 && page < num_pages && off >= 0 && off < page_size;
   if (hs >= heads + kv_heads) {                       // a value head: stored as it is
     const int hv = hs - heads - kv_heads;
     if (!page_ok) return;
-    const int64_t col = v_from_keys ? (int64_t)(heads + hv) * dim
-                                    : (int64_t)(heads + kv_heads) * dim + (int64_t)(hv / v_repeat) * vdim;
+    const int64_t col = v_from_keys ? (int64_t)(heads + hv) * dim : (int64_t)(heads + kv_heads) * dim + (int64_t)hv * vdim;
     const T* src = row + col;
     T* dst = pages + page * page_len + (int64_t)kv_heads * page_size * dim + (int64_t)hv * vdim * page_size + off;
     if (bias) {
@@ -179,17 +179,17 @@ extern "C" int holon_head_prepare(const void* qkv, void* q_out, int tokens, int 
                                   const void* q_weight, const void* k_weight, float eps, const float* table, int rot,
                                   int table_rows, const int32_t* positions, void* pages, const int32_t* write_page,
                                   const int32_t* write_off, int page_size, int num_pages, int dtype, const float* bias,
-                                  int stride, int v_from_keys, int v_repeat, void* stream) {
-  HOLON_CHECK(tokens >= 0 && heads > 0 && kv_heads >= 0 && dim > 0 && vdim > 0 && v_repeat >= 1 &&
-                  kv_heads % v_repeat == 0 && (!v_from_keys || (vdim == dim && v_repeat == 1)),
+                                  int stride, int v_from_keys, int v_share, void* stream) {
+  HOLON_CHECK(tokens >= 0 && heads > 0 && kv_heads >= 0 && dim > 0 && vdim > 0 && v_share >= 1 &&
+                  kv_heads % v_share == 0 && (!v_from_keys || (vdim == dim && v_share == 1)),
               "head_prepare: %d/%d heads of %d/%d, a value head for every %d key heads%s", heads, kv_heads, dim, vdim,
-              v_repeat, v_from_keys ? ", values from the keys" : "");
+              v_share, v_from_keys ? ", values from the keys" : "");
   HOLON_CHECK((table == nullptr && rot == 0) || (rot > 0 && rot % 2 == 0 && rot <= dim && table_rows > 0),
               "head_prepare: %d rotary dimensions for heads of %d", rot, dim);
   HOLON_CHECK((q_weight == nullptr) == (k_weight == nullptr), "head_prepare: one norm weight without the other");
   HOLON_CHECK(pages ? (kv_heads > 0 && page_size > 0 && num_pages > 0 && write_page && write_off) : kv_heads == 0,
               "head_prepare: bad page geometry, or key heads without pages to store them");
-  const int64_t width = (int64_t)(heads + kv_heads) * dim + (v_from_keys ? 0 : (int64_t)(kv_heads / v_repeat) * vdim);
+  const int64_t width = (int64_t)(heads + kv_heads) * dim + (v_from_keys ? 0 : (int64_t)(kv_heads / v_share) * vdim);
   HOLON_CHECK(stride >= width, "head_prepare: rows of %d values hold no %lld columns", stride, (long long)width);
   if (tokens == 0) return 0;
   HOLON_CHECK((heads + 2 * kv_heads + 3) / 4 <= 65535, "head_prepare: too many heads for one launch");
@@ -199,12 +199,12 @@ extern "C" int holon_head_prepare(const void* qkv, void* q_out, int tokens, int 
     head_prepare_kernel<float><<<grid, 256, 0, s>>>((const float*)qkv, (float*)q_out, heads, kv_heads, dim, vdim,
                                                     (const float*)q_weight, (const float*)k_weight, eps, table, rot,
                                                     table_rows, positions, (float*)pages, write_page, write_off,
-                                                    page_size, num_pages, bias, stride, v_from_keys, v_repeat);
+                                                    page_size, num_pages, bias, stride, v_from_keys, v_share);
   else
     head_prepare_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)qkv, (bf16_t*)q_out, heads, kv_heads, dim, vdim,
                                                      (const bf16_t*)q_weight, (const bf16_t*)k_weight, eps, table, rot,
                                                      table_rows, positions, (bf16_t*)pages, write_page, write_off,
-                                                     page_size, num_pages, bias, stride, v_from_keys, v_repeat);
+                                                     page_size, num_pages, bias, stride, v_from_keys, v_share);
   HOLON_LAUNCH_OK();
   return 0;
 }

@@ -5,7 +5,7 @@
 // visible (key j is seen if j <= i and (i - j < window or j < keep_first)).
 //
 // A page of one site holds P tokens: keys [Hkv, P, D] (a token's key is a row), then values [Hkv, V, P] (transposed
-// inside the page). One block of four waves per (token, head). Keys are walked in tiles of 64 that start at multiples
+// inside the page); with `v_share` s > 1 only Hkv / s value heads, key head h reading value head h / s. One block of four waves per (token, head). Keys are walked in tiles of 64 that start at multiples
 // of 64 (so a tile is whole pages wherever P divides 64), wave w taking tiles w, w + 4, ... of those the query sees (the
 // tiles of the kept first tokens, where they lie wholly before the window's first tile, then the window's); a
 // lane takes one key of a tile: its score over D, with the query in LDS. For the values the lanes turn to the value
@@ -26,7 +26,7 @@ __global__ void __launch_bounds__(256) softmax_attention_kernel(
     int table_stride, int table_rows, const int32_t* __restrict__ slots, const int32_t* __restrict__ token_row,
     const int32_t* __restrict__ positions, int heads, int kv_heads, int dim, int vdim, int page_size, int num_pages,
     const float* __restrict__ sink, float scale, int window, int key_vec, float softcap,
-    const float* __restrict__ r1, const float* __restrict__ r2, int keep_first) {
+    const float* __restrict__ r1, const float* __restrict__ r2, int keep_first, int v_share) {
   __shared__ float q_s[SMX_MAX_D];
   __shared__ float sum_s[4][SMX_MAX_D];
   __shared__ float ml_s[4][2];
@@ -37,8 +37,9 @@ __global__ void __launch_bounds__(256) softmax_attention_kernel(
   int slot = slots[token_row[t]];
   slot = slot < 0 ? 0 : (slot >= table_rows ? table_rows - 1 : slot);
   const int32_t* trow = table + (int64_t)slot * table_stride;
-  const int64_t page_len = (int64_t)kv_heads * page_size * (dim + vdim);
-  const int64_t val_base = (int64_t)kv_heads * page_size * dim + (int64_t)hk * vdim * page_size;
+  // (v_share key heads read one value head: a page then holds kv_heads / v_share value heads behind its keys)
+  const int64_t page_len = (int64_t)kv_heads * page_size * dim + (int64_t)(kv_heads / v_share) * page_size * vdim;
+  const int64_t val_base = (int64_t)kv_heads * page_size * dim + (int64_t)(hk / v_share) * vdim * page_size;
   const T* qp = q + ((int64_t)t * heads + h) * dim;
   for (int d = threadIdx.x; d < dim; d += 256) q_s[d] = Elem<T>::load(qp[d]);
   __syncthreads();
@@ -163,9 +164,11 @@ extern "C" int holon_softmax_attention(const void* q, void* out, const void* pag
                                        const int32_t* token_row, const int32_t* positions, int tokens, int heads,
                                        int kv_heads, int dim, int vdim, int page_size, int num_pages, const float* sink,
                                        float scale, int window, int dtype, float softcap, const float* r1,
-                                       const float* r2, int keep_first, void* stream) {
+                                       const float* r2, int keep_first, int v_share, void* stream) {
   HOLON_CHECK(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "softmax_attention: %d/%d heads", heads,
               kv_heads);
+  HOLON_CHECK(v_share >= 1 && kv_heads % v_share == 0, "softmax_attention: %d key heads do not share value heads by %d",
+              kv_heads, v_share);
   HOLON_CHECK(dim > 0 && dim <= SMX_MAX_D && vdim > 0 && vdim <= SMX_MAX_D,
               "softmax_attention: head sizes %d/%d (at most %d)", dim, vdim, SMX_MAX_D);
   HOLON_CHECK(page_size > 0 && num_pages > 0 && window >= 0 && table_stride > 0 && table_rows > 0,
@@ -184,7 +187,7 @@ extern "C" int holon_softmax_attention(const void* q, void* out, const void* pag
   softmax_attention_kernel<T, PV><<<grid, 256, 0, s>>>((const T*)q, (T*)out, (const T*)pages, table, table_stride,   \
                                                        table_rows, slots, token_row, positions, heads, kv_heads, dim, \
                                                        vdim, page_size, num_pages, sink, scale, window, key_vec,     \
-                                                       softcap, r1, r2, keep_first)
+                                                       softcap, r1, r2, keep_first, v_share)
   if (dtype == HOLON_F32) { if (paged_vec) SMX_LAUNCH(float, true); else SMX_LAUNCH(float, false); }
   else { if (paged_vec) SMX_LAUNCH(bf16_t, true); else SMX_LAUNCH(bf16_t, false); }
 #undef SMX_LAUNCH

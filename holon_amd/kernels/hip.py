@@ -82,6 +82,10 @@ class HipKernels:
                                                  _P, _F, _P, _P, _I, _P],
             "holon_attention_decode_mod_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
                                                 _P, _P, _I, _I, _I, _I, _P, _F, _P, _P, _I, _P],
+            "holon_attention_prefill_shared_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F,
+                                                    _I, _P, _F, _P, _P, _I, _I, _P],
+            "holon_attention_decode_shared_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
+                                                   _P, _P, _I, _I, _I, _I, _P, _F, _P, _P, _I, _I, _P],
             "holon_attention_decode_fused_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
                                                   _P, _P, _F, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P],
             "holon_gemm_skinny_supported": [_I, _I, _I],
@@ -643,11 +647,14 @@ class HipKernels:
         return bool(dtype in _DT and self.lib.holon_attention_mfma_supported(head_dim, page_size, _DT[dtype]))
 
     def paged_attention(self, q, pages, table, rows: AttnRows, page_size, scale, window, sink=None, softcap=0.0,
-                        dist=None, keep_first=0):
+                        dist=None, keep_first=0, value_share=1):
         self._check(q, "attention q")
         self._check(pages, "attention pages", q.dtype)
         self._check(table, "block table", torch.int32)
         t, hq, d = q.shape
+        if value_share > 1:
+            return self._shared_attention(q, pages, table, rows, page_size, scale, window, sink, softcap, dist,
+                                          keep_first, int(value_share))
         hkv = pages.shape[2]
         if pages.shape[1] != 2 or pages.shape[3] != page_size * d:
             raise KernelError(f"attention: pages {tuple(pages.shape)} do not fit head_dim {d}, page {page_size}")
@@ -707,6 +714,41 @@ class HipKernels:
                    table.shape[1], rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr(), b, t, hq,
                    hkv, d, page_size, pages.shape[0], float(scale), int(window), self._dt(q, "attention"),
                    self._stream())
+        return out
+
+    def _shared_attention(self, q, pages, table, rows, page_size, scale, window, sink, softcap, dist, keep_first, share):
+        """`paged_attention` over pages [n, Hkv + Hkv / share, P * D] whose key heads share value heads: the
+        matrix-core kernels alone (a caller asks `attention_on_cores` first)."""
+        t, hq, d = q.shape
+        if pages.dim() != 3 or pages.shape[2] != page_size * d or pages.shape[1] % (share + 1):
+            raise KernelError(f"attention: pages {tuple(pages.shape)} do not hold key heads that share value heads by "
+                              f"{share} at head_dim {d}, page {page_size}")
+        hkv = pages.shape[1] // (share + 1) * share
+        if not self.lib.holon_attention_mfma_supported(d, page_size, self._dt(q, "attention")) or hq % hkv:
+            raise KernelError(f"attention: shared value heads are served by the matrix-core kernels, not at head_dim "
+                              f"{d}, page {page_size}, {q.dtype}, {hq}/{hkv} heads")
+        for v in (sink,) + tuple(dist or ()):
+            if v is not None:
+                self._check(v, "attention sink or distance bias", torch.float32)
+                if v.shape != (hq,):
+                    raise KernelError(f"attention: {tuple(v.shape)} numbers for {hq} heads")
+        out = torch.empty_like(q)
+        common = (q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(), table.shape[1],
+                  rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr())
+        mod = (float(softcap), _ptr(dist[0]) if dist is not None else None,
+               _ptr(dist[1]) if dist is not None else None, int(keep_first) if window > 0 else 0, share)
+        if rows.n_chunk:
+            self._call(self.lib.holon_attention_prefill_shared_bf16, *common, rows.chunk_rows.data_ptr(), rows.n_chunk,
+                       rows.max_chunk_query, rows.max_chunk_len, hq, hkv, d, page_size, float(scale), int(window),
+                       _ptr(sink), *mod, self._stream())
+        if rows.n_decode:
+            span = rows.max_decode_len if not window else min(rows.max_decode_len, window + 31)
+            splits, per, waves = self.decode_splits(rows.n_decode * hkv * ((hq // hkv + 15) // 16), span, d)
+            part_o, part_ml = self._decode_parts(rows.n_decode * hq * (splits // waves), d, q.device)
+            self._call(self.lib.holon_attention_decode_shared_bf16, *common, rows.decode_rows.data_ptr(),
+                       rows.n_decode, rows.max_decode_len, hq, hkv, d, page_size, float(scale), int(window),
+                       _ptr(part_o), _ptr(part_ml), splits, per, waves, int(rows.in_order and rows.n_decode == t),
+                       _ptr(sink), *mod, self._stream())
         return out
 
     def qkv_attention(self, qkv, heads, kv_heads, head_dim, q_weight, k_weight, eps, rope_table, positions, pages,

@@ -7,9 +7,9 @@ square and multiplied by a constant:
 The two maps are two ordinary softmax attentions, so the mixer hands the framework's attention kernels 2H query heads
 over 2G key heads: the query projection's rows are reordered once after loading from (head, map) to (kv head, map, head
 within the group), so that the kernels' grouping, query head // (H / G), sends map m of a head to map m of its kv
-head; a key head's value head is kv head // 2 in the design and is stored once for each map, so that every kernel
-reads a page as it reads any other (the price: G vdim more values a token than the design needs). `diff_combine` puts
-the maps together and brings the heads back into the design's order.
+head. Key head (kv head, map) reads value head kv head: a page holds the 2G key heads and behind them the G value
+heads, once, and the attention kernels are told that two key heads share a value head (`value_share=2`).
+`diff_combine` puts the maps together and brings the heads back into the design's order.
 
 Queries and keys are RMS-normed per head and map with one weight of `dim` values each (`q_norm`, `k_norm`) and turned
 by a registered position part (one that says `interleaved` has the rows of both projections, and the norms' weights,
@@ -97,8 +97,8 @@ class DiffAttention(Part):
         self.lam: float | None = None
 
     def state(self):
-        # keys of both maps and the values once for each map, for every kv head
-        return [PagedState(self.state_name, elems=2 * self.kv_heads * (self.dim + self.vdim))]
+        # the keys of both maps and the values, for every kv head
+        return [PagedState(self.state_name, elems=self.kv_heads * (2 * self.dim + self.vdim))]
 
     def finalize(self) -> None:
         if self.q.weight is None:
@@ -143,11 +143,11 @@ class DiffAttention(Part):
         if self.own_kv:
             q = k.head_prepare(self.qkv(x), 2 * self.heads, 2 * self.kv_heads, self.dim, self.vdim, self.q_norm,
                                self.k_norm, self.eps, table, step.positions, held.pages, view.write_page,
-                               view.write_off, view.page_size, value_repeat=2)
+                               view.write_off, view.page_size, value_share=2)
         else:
             q = k.head_prepare(self.qkv(x), 2 * self.heads, 0, self.dim, self.vdim, self.q_norm, self.q_norm,
                                self.eps, table, step.positions, None, None, None, view.page_size)
-        maps = attend(k, q, held, view, step, 2 * self.kv_heads, self.vdim, None, self.scale, 0)
+        maps = attend(k, q, held, view, step, 2 * self.kv_heads, self.vdim, None, self.scale, 0, value_share=2)
         return self.o(k.diff_combine(maps, self.heads, self.kv_heads, self.vdim, self.lam, self.eps, 1.0 - self.diff))
 
     __call__ = forward

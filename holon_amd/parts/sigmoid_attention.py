@@ -28,23 +28,23 @@ def _ptr(t):
 
 
 def head_prepare_plain(qkv, heads, kv_heads, dim, vdim, q_weight, k_weight, eps, table, positions, pages, write_page,
-                       write_off, page_size, bias=None, values="own", value_repeat=1):
+                       write_off, page_size, bias=None, values="own", value_share=1):
     """qkv [T, >= (H + G) D + G' V] (queries, keys, values side by side in the first columns of every row; a row may
     hold more behind them); `bias` (float32, one value a column of q, k and v, or None) is added first. Per head of q
     and k: x * rsqrt(mean(x^2) + eps)
     * weight (when weights are given), then the rotation by `table` [positions, rot] (cos of rot/2 angles, then
     their sines; pairs (i, i + rot/2); dimensions from rot on pass), all in float32 with one rounding. Keys and
-    values go into `pages` [pages, G P (D + V)] (keys [G, P, D], then values [G, V, P]) at (write_page[t],
+    values go into `pages` [pages, G P D + G' P V] (keys [G, P, D], then values [G', V, P]) at (write_page[t],
     write_off[t]); returns q [T, H, D].
 
-    Where the values come from: `values` "own": the G' = G / value_repeat value heads behind the keys, cache value head
-    g being projected head g // value_repeat (several key heads over one value head); "keys": there are no value
-    columns and value head g is key head g as projected (bias added; before the norm and the rotation), V = D.
+    Where the values come from: `values` "own": the G' = G / value_share value heads behind the keys (`value_share`
+    key heads read one value head; the page holds G' value heads); "keys": there are no value columns and value head g
+    is key head g as projected (bias added; before the norm and the rotation), V = D and G' = G.
     `pages` None: the rows hold queries alone (H D columns) and nothing is stored."""
     t, out_dtype = qkv.shape[0], qkv.dtype
     if pages is None:
         kv_heads = 0
-    shared = kv_heads // value_repeat if values == "own" else 0
+    shared = kv_heads // value_share if values == "own" else 0
     width = (heads + kv_heads) * dim + shared * vdim
     qkv = qkv[:, :width]
     if bias is not None:
@@ -52,7 +52,7 @@ def head_prepare_plain(qkv, heads, kv_heads, dim, vdim, q_weight, k_weight, eps,
     q = qkv[:, : heads * dim].float().view(t, heads, dim)
     k = qkv[:, heads * dim: (heads + kv_heads) * dim].float().view(t, kv_heads, dim)
     if values == "own":
-        v = qkv[:, (heads + kv_heads) * dim:].reshape(t, shared, vdim).repeat_interleave(value_repeat, dim=1)
+        v = qkv[:, (heads + kv_heads) * dim:].reshape(t, shared, vdim)
     else:
         v = k.clone()
     if q_weight is not None:
@@ -70,25 +70,26 @@ def head_prepare_plain(qkv, heads, kv_heads, dim, vdim, q_weight, k_weight, eps,
     if pages is None:
         return q.to(out_dtype)
     keys = pages[:, : kv_heads * page_size * dim].view(-1, kv_heads, page_size, dim)
-    vals = pages[:, kv_heads * page_size * dim:].view(-1, kv_heads, vdim, page_size)
+    vals = pages[:, kv_heads * page_size * dim:].view(-1, v.shape[1], vdim, page_size)
     keys[write_page[:t].long(), :, write_off[:t].long()] = k.to(pages.dtype)
     vals[write_page[:t].long(), :, :, write_off[:t].long()] = v.to(pages.dtype)
     return q.to(pages.dtype)
 
 
 def _head_prepare_hip(launch, qkv, heads, kv_heads, dim, vdim, q_weight, k_weight, eps, table, positions, pages,
-                      write_page, write_off, page_size, bias=None, values="own", value_repeat=1):
+                      write_page, write_off, page_size, bias=None, values="own", value_share=1):
     t, stride = qkv.shape
     if pages is None:
         kv_heads = 0
     from_keys = values == "keys"
-    ok = values in ("own", "keys") and value_repeat >= 1 and kv_heads % value_repeat == 0 \
-        and (not from_keys or (vdim == dim and value_repeat == 1))
-    shared = kv_heads // value_repeat if ok and not from_keys else 0
+    ok = values in ("own", "keys") and value_share >= 1 and kv_heads % value_share == 0 \
+        and (not from_keys or (vdim == dim and value_share == 1))
+    shared = kv_heads // value_share if ok and not from_keys else 0
     width = (heads + kv_heads) * dim + shared * vdim
     ok = ok and qkv.is_cuda and qkv.is_contiguous() and qkv.dtype in _DT and stride >= width \
         and (pages is None or (pages.dtype == qkv.dtype and pages.is_contiguous() and pages.dim() == 2
-                               and pages.shape[1] == kv_heads * page_size * (dim + vdim)
+                               and pages.shape[1] == kv_heads * page_size * dim
+                               + (kv_heads if from_keys else shared) * page_size * vdim
                                and write_page.shape[0] >= t and write_off.shape[0] >= t)) \
         and (q_weight is None) == (k_weight is None) \
         and all(w is None or (w.dtype == qkv.dtype and w.shape == (dim,)) for w in (q_weight, k_weight)) \
@@ -99,7 +100,7 @@ def _head_prepare_hip(launch, qkv, heads, kv_heads, dim, vdim, q_weight, k_weigh
     if not ok:
         raise ValueError(f"head_prepare: qkv {tuple(qkv.shape)} {qkv.dtype}, pages "
                          f"{None if pages is None else tuple(pages.shape)} do not fit {heads}/{kv_heads} heads of "
-                         f"{dim}/{vdim}, page {page_size}, values {values!r} x{value_repeat}")
+                         f"{dim}/{vdim}, page {page_size}, values {values!r} shared by {value_share}")
     q = torch.empty((t, heads, dim), dtype=qkv.dtype, device=qkv.device)
     if t:
         launch(qkv.data_ptr(), q.data_ptr(), t, heads, kv_heads, dim, vdim, _ptr(q_weight), _ptr(k_weight), float(eps),
@@ -107,7 +108,7 @@ def _head_prepare_hip(launch, qkv, heads, kv_heads, dim, vdim, q_weight, k_weigh
                positions.data_ptr(), _ptr(pages), _ptr(write_page) if pages is not None else None,
                _ptr(write_off) if pages is not None else None, page_size,
                pages.shape[0] if pages is not None else 0, _DT[qkv.dtype], _ptr(bias), stride, 1 if from_keys else 0,
-               int(value_repeat))
+               int(value_share))
     return q
 
 

@@ -30,17 +30,20 @@ def _ptr(t):
 
 
 def softmax_attention_plain(q, pages, table, rows, token_row, positions, kv_heads, vdim, page_size, sink, scale,
-                            window, softcap=0.0, dist=None, keep_first=0):
+                            window, softcap=0.0, dist=None, keep_first=0, value_share=1):
     """q [T, H, D]; `pages` [pages, G P (D + V)] (keys [G, P, D], then values [G, V, P]); `table` [S, max_pages]
     int32; token t belongs to row token_row[t] (slot rows.slots[row]) and stands at positions[t]. Query at position p
     sees keys max(0, p - window + 1) .. p (window 0: 0 .. p). weights = exp(s_j - top) / (sum_j exp(s_j - top) +
     exp(sink[h] - top)) with s = q . k * scale, `sink` [H] float32 or None (then no such term). With a window and
     `keep_first` > 0 the query also sees keys 0 .. keep_first - 1, at their true positions. `softcap` > 0: s <-
     softcap tanh(s / softcap); `dist` = (r1 [H], r2 [H]) float32: then s <- s - r1 ln(1 + r2 (p - j)) for the key at
-    position j. -> [T, H V] in q's dtype; scores, weights and sums in float32."""
+    position j. `value_share` s > 1: a page holds G / s value heads behind its G key heads, and key head g reads value
+    head g // s. -> [T, H V] in q's dtype; scores, weights and sums in float32."""
     t, heads, dim = q.shape
     keys = pages[:, : kv_heads * page_size * dim].view(-1, kv_heads, page_size, dim)
-    vals = pages[:, kv_heads * page_size * dim:].view(-1, kv_heads, vdim, page_size).transpose(2, 3)
+    vals = pages[:, kv_heads * page_size * dim:].view(-1, kv_heads // value_share, vdim, page_size).transpose(2, 3)
+    if value_share > 1:
+        vals = vals.repeat_interleave(value_share, dim=1)
     out = torch.zeros((t, heads, vdim), dtype=torch.float32, device=q.device)
     pos = positions.tolist()
     slot_of, row_of = rows.slots.tolist(), token_row.tolist()
@@ -71,13 +74,15 @@ def softmax_attention_plain(q, pages, table, rows, token_row, positions, kv_head
 
 
 def _softmax_attention_hip(launch, q, pages, table, rows, token_row, positions, kv_heads, vdim, page_size, sink,
-                           scale, window, softcap=0.0, dist=None, keep_first=0):
+                           scale, window, softcap=0.0, dist=None, keep_first=0, value_share=1):
     t, heads, dim = q.shape
     if dist is not None and not all(d.is_cuda and d.dtype == torch.float32 and d.is_contiguous() and d.shape == (heads,)
                                     for d in dist):
         raise ValueError("softmax_attention: the distance bias is two float32 numbers a head")
     ok = q.is_cuda and q.is_contiguous() and q.dtype in _DT and pages.dtype == q.dtype and pages.is_contiguous() \
-        and pages.dim() == 2 and pages.shape[1] == kv_heads * page_size * (dim + vdim) and table.dtype == torch.int32 \
+        and pages.dim() == 2 and value_share >= 1 and kv_heads % value_share == 0 \
+        and pages.shape[1] == kv_heads * page_size * dim + kv_heads // value_share * page_size * vdim \
+        and table.dtype == torch.int32 \
         and table.is_contiguous() and heads % kv_heads == 0 and token_row.shape[0] >= t and positions.shape[0] >= t \
         and (sink is None or (sink.dtype == torch.float32 and sink.is_contiguous() and sink.shape == (heads,)))
     if not ok:
@@ -87,7 +92,8 @@ def _softmax_attention_hip(launch, q, pages, table, rows, token_row, positions, 
     launch(q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(), table.shape[1], table.shape[0],
            rows.slots.data_ptr(), token_row.data_ptr(), positions.data_ptr(), t, heads, kv_heads, dim, vdim, page_size,
            pages.shape[0], _ptr(sink), float(scale), int(window), _DT[q.dtype], float(softcap),
-           _ptr(dist[0]) if dist is not None else None, _ptr(dist[1]) if dist is not None else None, int(keep_first))
+           _ptr(dist[0]) if dist is not None else None, _ptr(dist[1]) if dist is not None else None, int(keep_first),
+           int(value_share))
     return out
 
 
@@ -289,7 +295,7 @@ def _add_bias_hip(launch, x, bias):
 
 
 register_kernel(KernelOp("softmax_attention", softmax_attention_plain, "holon_softmax_attention",
-                         [_P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _I, _F, _P, _P, _I],
+                         [_P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _I, _F, _P, _P, _I, _I],
                          _softmax_attention_hip))
 register_kernel(KernelOp("head_linear", head_linear_plain, "holon_head_linear_rows",
                          [_P, _P, _P, _I, _I, _I, _I, _I, _I], _head_linear_hip))
@@ -304,18 +310,28 @@ register_kernel(KernelOp("head_gate", head_gate_plain, "holon_head_gate", [_P, _
 register_kernel(KernelOp("add_bias", add_bias_plain, "holon_add_bias", [_P, _P, _L, _I, _I], _add_bias_hip))
 
 
-def attend(k, q, held, view, step, kv_heads, vdim, sink, scale, window, softcap=0.0, dist=None, keep_first=0):
-    """The attention of both mixers: on the matrix cores where keys and values have one width that those kernels
-    serve (the pages' layout is then theirs), else the general kernel. q [T, H, D] -> [T, H V]."""
+def attend(k, q, held, view, step, kv_heads, vdim, sink, scale, window, softcap=0.0, dist=None, keep_first=0,
+           value_share=1):
+    """The attention of the mixers: on the matrix cores where keys and values have one width that those kernels
+    serve (the pages' layout is then theirs), else the general kernel. q [T, H, D] -> [T, H V]. `value_share` s > 1:
+    a page holds kv_heads / s value heads behind its kv_heads key heads, and key head g reads value head g // s."""
     t, heads, dim = q.shape
+    keep = keep_first if window > 0 else 0
     if dim == vdim and k.attention_on_cores(dim, view.page_size, q.dtype):
+        if value_share > 1:
+            pages = held.pages.view(-1, kv_heads + kv_heads // value_share, view.page_size * dim)
+            return k.paged_attention(q, pages, view.table, step.rows, view.page_size, scale, window, sink=sink,
+                                     softcap=softcap, dist=dist, keep_first=keep, value_share=value_share
+                                     ).view(t, heads * vdim)
         pages = held.pages.view(-1, 2, kv_heads, view.page_size * dim)
         return k.paged_attention(q, pages, view.table, step.rows, view.page_size, scale, window, sink=sink,
-                                 softcap=softcap, dist=dist, keep_first=keep_first if window > 0 else 0
-                                 ).view(t, heads * vdim)
+                                 softcap=softcap, dist=dist, keep_first=keep).view(t, heads * vdim)
+    if value_share > 1:
+        return k.softmax_attention(q, held.pages, view.table, step.rows, step.token_row, step.positions, kv_heads, vdim,
+                                   view.page_size, sink, scale, window, softcap=softcap, dist=dist, keep_first=keep,
+                                   value_share=value_share)
     return k.softmax_attention(q, held.pages, view.table, step.rows, step.token_row, step.positions, kv_heads, vdim,
-                               view.page_size, sink, scale, window, softcap=softcap, dist=dist,
-                               keep_first=keep_first if window > 0 else 0)
+                               view.page_size, sink, scale, window, softcap=softcap, dist=dist, keep_first=keep)
 
 
 def to_half_split(rows_per_head: int, heads: int, rot: int) -> torch.Tensor:

@@ -171,11 +171,16 @@ class TorchKernels:
         return self.cores
 
     def paged_attention(self, q, pages, table, rows, page_size, scale, window, sink=None, softcap=0.0, dist=None,
-                        keep_first=0):
+                        keep_first=0, value_share=1):
         t, hq, d = q.shape
-        hkv = pages.shape[2]
-        kp = pages[:, 0].view(-1, hkv, page_size, d)
-        vp = pages[:, 1].view(-1, hkv, d, page_size)
+        if value_share > 1:                  # [n, Hkv + Hkv / s, P D]: key head h reads value head h // s
+            hkv = pages.shape[1] // (value_share + 1) * value_share
+            kp = pages[:, :hkv].view(-1, hkv, page_size, d)
+            vp = pages[:, hkv:].view(-1, hkv // value_share, d, page_size).repeat_interleave(value_share, dim=1)
+        else:
+            hkv = pages.shape[2]
+            kp = pages[:, 0].view(-1, hkv, page_size, d)
+            vp = pages[:, 1].view(-1, hkv, d, page_size)
         out = torch.zeros_like(q)
         qs = rows.query_start.tolist()
         for b, (slot, n) in enumerate(zip(rows.slots.tolist(), rows.lens.tolist())):

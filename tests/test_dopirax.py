@@ -551,22 +551,22 @@ def test_kernels_alone_against_their_plain_forms(dtype):
     write_off = (positions % page).to(torch.int32)
     total = sum(lens)
     prepare = kernel_op("head_prepare").plain
-    for heads, groups, dim, vdim, rot, values, repeat, extra, normed, biased in (
+    for heads, groups, dim, vdim, rot, values, share, extra, normed, biased in (
             (4, 2, 24, 24, 12, "keys", 1, 16, False, True), (6, 4, 16, 40, 8, "own", 2, 0, True, False),
             (4, 2, 64, 64, 64, "own", 2, 3, True, False), (3, 3, 8, 8, 0, "keys", 1, 0, False, False),
             (4, 4, 16, 12, 16, "own", 1, 0, True, True)):
-        shared = groups // repeat if values == "own" else 0
+        shared = groups // share if values == "own" else 0
         width = (heads + groups) * dim + shared * vdim
         qkv = randn(total, width + extra)
         tab = rope_table(256, rot, 1000.0).to(dev) if rot else None
         qw = (1 + 0.2 * randn(dim, to=torch.float32)).to(dtype) if normed else None
         kw = (1 + 0.2 * randn(dim, to=torch.float32)).to(dtype) if normed else None
         bias = randn(width, to=torch.float32) if biased else None
-        pa = torch.zeros(n_pages, groups * page * (dim + vdim), device=dev, dtype=dtype)
+        pa = torch.zeros(n_pages, groups * page * dim + (shared or groups) * page * vdim, device=dev, dtype=dtype)
         pb = pa.clone()
         args = (heads, groups, dim, vdim, qw, kw, 1e-6, tab, positions)
-        qa = k.head_prepare(qkv, *args, pa, write_page, write_off, page, bias=bias, values=values, value_repeat=repeat)
-        qb = prepare(qkv, *args, pb, write_page, write_off, page, bias=bias, values=values, value_repeat=repeat)
+        qa = k.head_prepare(qkv, *args, pa, write_page, write_off, page, bias=bias, values=values, value_share=share)
+        qb = prepare(qkv, *args, pb, write_page, write_off, page, bias=bias, values=values, value_share=share)
         assert H.rel_rms(qa, qb) < tol and H.rel_rms(pa, pb) < tol, (heads, groups, dim, values)
         only_q = qkv[:, : heads * dim].contiguous()
         qa = k.head_prepare(only_q, heads, 0, dim, vdim, qw, kw, 1e-6, tab, positions, None, None, None, page,
