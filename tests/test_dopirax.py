@@ -638,3 +638,57 @@ def test_the_cap_and_the_fixed_sink_on_the_matrix_cores(dim):
         assert H.rel_rms(got, want) < 8e-3, (dim, scale, cap)
         per = ((got.double() - want).square().mean((1, 2)).sqrt() / want.square().mean().sqrt()).max().item()
         assert per < 4e-2, (dim, scale, cap, per)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dim", [64, 128, 256])
+def test_key_heads_that_share_value_heads_on_the_gpu(dim):
+    """Pages that hold fewer value heads than key heads (two or three key heads read one value head): the matrix-core
+    prompt and decode kernels in bfloat16 and the general kernel in both types, prompt portions beside decode rows over
+    scattered pages, with and without a sink and a cap, against float64."""
+    import holon_amd.parts  # noqa: F401
+    from holon_amd.kernels import load_hip
+    from holon_amd.kernels.api import AttnRows
+    from holon_amd.kernels.registry import kernel_op
+    k, dev, page = load_hip(), "cuda", 16
+    g = torch.Generator().manual_seed(dim + 2)
+    lens, counts = [300, 75, 190, 3, 129, 1, 40], [300, 1, 60, 3, 1, 1, 2]
+    n_pages = sum(-(-n // page) for n in lens) + 1
+    table = torch.full((len(lens) + 1, 24), n_pages - 1, dtype=torch.int32)
+    order, at = torch.randperm(n_pages - 1, generator=g).tolist(), 0
+    for s_, n in enumerate(lens):
+        for i in range(-(-n // page)):
+            table[s_, i] = order[at]
+            at += 1
+    qstart = [0]
+    for c in counts:
+        qstart.append(qstart[-1] + c)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)          # noqa: E731
+    decode = [b for b, c in enumerate(counts) if c == 1]
+    chunk = [b for b, c in enumerate(counts) if c > 1]
+    rows = AttnRows(slots=i32(list(range(len(lens)))), lens=i32(lens), query_start=i32(qstart), decode_rows=i32(decode),
+                    chunk_rows=i32(chunk), n_decode=len(decode), n_chunk=len(chunk),
+                    max_decode_len=max(lens[b] for b in decode), max_chunk_query=max(counts),
+                    max_chunk_len=max(lens[b] for b in chunk))
+    token_row = torch.cat([torch.full((c,), b, dtype=torch.int32) for b, c in enumerate(counts)]).to(dev)
+    positions = torch.cat([torch.arange(n - c, n, dtype=torch.int32) for n, c in zip(lens, counts)]).to(dev)
+    twin, scale = TorchKernels(), 1.5 * dim ** -0.5
+    for heads, groups, share in ((8, 4, 2), (6, 6, 3), (12, 2, 2)):
+        pages = (torch.randn(n_pages, groups + groups // share, page * dim, generator=g) * 0.5).to(dev).bfloat16()
+        q = torch.randn(qstart[-1], heads, dim, generator=g).to(dev).bfloat16()
+        sink = torch.zeros(heads, device=dev)
+        for sk, cap in ((None, 0.0), (sink, 0.0), (sink, 4.0)):
+            want = twin.paged_attention(q.double(), pages.double(), table.to(dev), rows, page, scale, 0,
+                                        sink=None if sk is None else sk.double(), softcap=cap, value_share=share)
+            got = k.paged_attention(q, pages, table.to(dev), rows, page, scale, 0, sink=sk, softcap=cap, value_share=share)
+            assert H.rel_rms(got, want) < 8e-3, (dim, heads, groups, share, cap)
+            per = ((got.double() - want).square().mean((1, 2)).sqrt() / want.square().mean().sqrt()).max().item()
+            assert per < 4e-2, (dim, heads, groups, share, cap, per)
+            flat = pages.view(n_pages, -1)
+            for dtype, tol in ((torch.bfloat16, 8e-3), (torch.float32, 2e-6)):
+                ref = want if dtype == torch.bfloat16 else kernel_op("softmax_attention").plain(
+                    q.double(), flat.double(), table.to(dev), rows, token_row, positions, groups, dim, page,
+                    None if sk is None else sk.double(), scale, 0, softcap=cap, value_share=share).view(-1, heads, dim)
+                general = k.softmax_attention(q.to(dtype), flat.to(dtype), table.to(dev), rows, token_row, positions,
+                                              groups, dim, page, sk, scale, 0, softcap=cap, value_share=share)
+                assert H.rel_rms(general.view(-1, heads, dim), ref) < tol, (dim, heads, groups, share, cap, dtype)
