@@ -69,11 +69,18 @@ class DopiraxConfig:
         layers = _get(c, "layers")
         if not isinstance(layers, list) or not layers:
             raise ConfigError("`layers` must be a non-empty list")
+        layers = json.loads(json.dumps(layers))            # a copy: defaults are filled in below
         for i, layer in enumerate(layers):
             at = f"layers[{i}]"
             kind, m = _get(layer, "type"), _get(layer, "mixer")
             if kind not in MIXERS:
                 raise ConfigError(f"{at}: unknown layer type {kind!r} ({', '.join(MIXERS)})")
+            if not isinstance(m, Mapping):
+                raise ConfigError(f"{at}: `mixer` must hold the mixer's sizes")
+            if kind == "attention" and "dim" in m:
+                m.setdefault("vdim", m["dim"])             # the values are the keys
+            if "heads" in m:
+                m.setdefault("kv_heads", m["heads"])       # no grouping named: every head has its own keys
             for key in ("heads", "kv_heads", "dim", "vdim"):
                 _get(m, key, int)
             _get(m, "scale", float)
@@ -99,7 +106,7 @@ class DopiraxConfig:
                         raise ConfigError(f"{at}: layer {src}'s kv_heads, dim, vdim and rot must equal this layer's")
             if layer.get("mlp"):
                 _check_mlp(at, layer["mlp"])
-        return cls(width=width, vocab=vocab, eps=eps, embedding_scale=scale, layers=tuple(json.loads(json.dumps(layers))),
+        return cls(width=width, vocab=vocab, eps=eps, embedding_scale=scale, layers=tuple(layers),
                    eos_token_ids=eos_ids(c, generation))
 
     def to_dict(self) -> dict[str, Any]:

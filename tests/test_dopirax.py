@@ -379,6 +379,9 @@ def test_configuration_and_weights_are_checked(tmp_path):
     cfg, spec = resolve(M.CONFIG_A)
     assert [(r.layer, r.reads) for r in spec.order] == [(0, None), (1, None), (2, 1), (3, None), (4, 1)]
     assert cfg.to_dict()["layers"] == M.CONFIG_A["layers"]
+    bare = M.variant(M.CONFIG_A)                                # sizes a configuration may leave to the design
+    del bare["layers"][0]["mixer"]["vdim"], bare["layers"][3]["mixer"]["kv_heads"]
+    assert resolve(bare)[0].to_dict()["layers"] == M.CONFIG_A["layers"] and "vdim" not in bare["layers"][0]["mixer"]
     late = M.variant(M.CONFIG_A)
     late["layers"][2]["mixer"]["kv_from"] = 3                   # an attention layer, and not an earlier one
     chain = M.variant(M.CONFIG_A)
