@@ -72,6 +72,10 @@ struct AttnArgs {
   const float* r1;
   const float* r2;
   int keep_first;
+  // one gate a (token, head) (nullable; row t of it starts at hgate + t * hgate_stride): head h's result of token t is
+  // multiplied by sigmoid(hgate[t, h]), which the kernels take as a factor 1 + exp(-gate) of the softmax's denominator
+  const bf16_t* hgate;
+  int64_t hgate_stride;
   // key heads that share one value head (0 or 1: every key head has its own): a page then holds kv_heads planes of
   // keys and kv_heads / v_share planes of values, and key head hk reads value head hk / v_share
   int v_share;
@@ -92,9 +96,10 @@ struct ModLane {
 
 // The denominator of a row whose keys summed to `l` under the running maximum `m` (in units of log2): with a sink, its
 // term beside them. A row that saw no key (m = -inf) keeps l = 0 and its result of zero.
-__device__ __forceinline__ float with_sink(const AttnArgs& a, int head, float l, float m) {
-  if (a.sink == nullptr || m == -INFINITY) return l;
-  return l + exp2f(a.sink[head] * 1.4426950408889634f - m);
+__device__ __forceinline__ float with_sink(const AttnArgs& a, int token, int head, float l, float m) {
+  if (a.sink != nullptr && m != -INFINITY) l += exp2f(a.sink[head] * 1.4426950408889634f - m);
+  if (a.hgate != nullptr) l *= 1.0f + __expf(-bf16_to_float(a.hgate[(int64_t)token * a.hgate_stride + head]));
+  return l;
 }
 
 // How the 16 rows of a tile map to (position, head) for a group of G heads.
@@ -432,7 +437,7 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
     lt += __shfl_xor(lt, 16, WAVE);
     lt += __shfl_xor(lt, 32, WAVE);
     if (!rr[t].valid) continue;
-    lt = with_sink(a, rr[t].head, lt, m[t]);
+    lt = with_sink(a, rr[t].token, rr[t].head, lt, m[t]);
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     bf16_t* op = a.out + ((int64_t)rr[t].token * a.heads + rr[t].head) * D + 4 * g;
 #pragma unroll
@@ -638,7 +643,7 @@ __global__ void __launch_bounds__(256) attn_prefill_lds_kernel(AttnArgs a) {
       lt += __shfl_xor(lt, 16, WAVE);
       lt += __shfl_xor(lt, 32, WAVE);
       if (!rr[t].valid) continue;
-      lt = with_sink(a, rr[t].head, lt, m[t]);
+      lt = with_sink(a, rr[t].token, rr[t].head, lt, m[t]);
       const float inv = lt > 0.f ? 1.0f / lt : 0.f;
       bf16_t* op = a.out + ((int64_t)rr[t].token * a.heads + rr[t].head) * D + 4 * g;
 #pragma unroll
@@ -910,7 +915,7 @@ __global__ void __launch_bounds__(256, D == 128 ? 2 : 3) attn_prefill_wide_kerne
     }
     float lt = l + __shfl_xor(l, 32, WAVE);
     if (valid) {
-      if (!SIG) lt = with_sink(a, head, lt, m);
+      if (!SIG) lt = with_sink(a, token, head, lt, m);
       const float inv = SIG ? 1.0f : (lt > 0.f ? 1.0f / lt : 0.f);
       bf16_t* op = a.out + ((int64_t)token * a.heads + head) * D + 4 * h;
       const bf16_t* gp = SIG && a.gate ? a.gate + ((int64_t)token * a.heads + head) * D + 4 * h : nullptr;
@@ -1205,7 +1210,7 @@ __global__ void __launch_bounds__(256, 2) attn_prefill_dma_kernel(AttnArgs a) {
     stage(std::true_type{}, kb_last, buf);
     float lt = l + __shfl_xor(l, 32, WAVE);
     if (valid) {
-      lt = with_sink(a, head, lt, m);
+      lt = with_sink(a, token, head, lt, m);
       const float inv = lt > 0.f ? 1.0f / lt : 0.f;
       bf16_t* op = a.out + ((int64_t)token * a.heads + head) * D + 4 * h;
 #pragma unroll
@@ -1452,7 +1457,7 @@ __global__ void __launch_bounds__(256, 1) attn_prefill_pair_kernel(AttnArgs a) {
     for (int t = 0; t < 2; ++t) {
       float lt = l[t] + __shfl_xor(l[t], 32, WAVE);
       if (valid[t]) {
-        lt = with_sink(a, head, lt, m[t]);
+        lt = with_sink(a, token[t], head, lt, m[t]);
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
         bf16_t* op = a.out + ((int64_t)token[t] * a.heads + head) * D + 4 * h;
 #pragma unroll
@@ -1732,7 +1737,7 @@ __global__ void __launch_bounds__(512) attn_decode_kernel(AttnArgs a, FusedArgs 
   }
   if (wave == 0 && rr.valid) {
     if (a.out_splits == 1) {             // the row's whole result: normalised and rounded here
-      if (!SIG) lt = with_sink(a, rr.head, lt, mt);
+      if (!SIG) lt = with_sink(a, rr.token, rr.head, lt, mt);
       const float inv = SIG ? 1.0f : (lt > 0.f ? 1.0f / lt : 0.f);
       bf16_t* op = a.out + ((int64_t)rr.token * a.heads + rr.head) * D + 4 * g;
       const bf16_t* gp = SIG && a.gate ? a.gate + ((int64_t)rr.token * a.heads + rr.head) * D + 4 * g : nullptr;
@@ -1775,7 +1780,9 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict
                                                          const float* __restrict__ part_ml, bf16_t* __restrict__ out,
                                                          const int32_t* __restrict__ row_ids,
                                                          const int32_t* __restrict__ qstart, int heads, int splits,
-                                                         const float* __restrict__ sink) {
+                                                         const float* __restrict__ sink,
+                                                         const bf16_t* __restrict__ hgate = nullptr,
+                                                         int64_t hgate_stride = 0) {
   constexpr int LANES = D / 4;            // threads across one partial
   constexpr int NG = 256 / LANES;         // groups of splits
   constexpr int PER = (64 + NG - 1) / NG; // splits a thread may own
@@ -1804,6 +1811,7 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict
     float denom = 0.f;                     // in split order
     for (int s = 0; s < splits; ++s) denom += __shfl(w_s * l_s, s, WAVE);
     if (sink != nullptr && big != -INFINITY) denom += exp2f(sink[h] * 1.4426950408889634f - big);
+    if (hgate != nullptr) denom *= 1.0f + __expf(-bf16_to_float(hgate[(int64_t)token * hgate_stride + h]));
     weight[tid] = w_s;
     if (tid == 0) inv_denom = denom > 0.f ? 1.0f / denom : 0.f;
   }
@@ -1882,7 +1890,7 @@ static int prefill_launch(const void* q, void* out, const void* pages, const int
                           const int32_t* slots, const int32_t* lens, const int32_t* query_start, const int32_t* row_ids,
                           int n_rows, int max_query, int max_len, int heads, int kv_heads, int head_dim, int page_size,
                           float scale, int window, const float* sink, void* stream, const ScoreMod* mod = nullptr,
-                          int v_share = 1) {
+                          int v_share = 1, const void* hgate = nullptr, int64_t hgate_stride = 0) {
   HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
@@ -1891,7 +1899,7 @@ static int prefill_launch(const void* q, void* out, const void* pages, const int
               v_share);
   if (n_rows <= 0 || max_query <= 0) return 0;
   AttnArgs a{};
-  a.v_share = v_share;
+  a.v_share = v_share; a.hgate = (const bf16_t*)hgate; a.hgate_stride = hgate_stride;
   a.q = (const bf16_t*)q; a.out = (bf16_t*)out; a.pages = (const bf16_t*)pages; a.table = table;
   a.table_stride = table_stride; a.slots = slots; a.lens = lens; a.qstart = query_start; a.row_ids = row_ids;
   a.heads = heads; a.kv_heads = kv_heads; a.page_size = page_size;
@@ -2054,13 +2062,16 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
                          int n_rows, int max_len, int heads, int kv_heads, int head_dim, int page_size, float scale,
                          int window, float* part_o, float* part_ml, int splits, int keys_per_split, void* stream,
                          const FusedArgs* fused = nullptr, int waves = 1, int rows_in_order = 0,
-                         const float* sink = nullptr, const ScoreMod* mod = nullptr, int v_share = 1) {
+                         const float* sink = nullptr, const ScoreMod* mod = nullptr, int v_share = 1,
+                         const void* hgate = nullptr, int64_t hgate_stride = 0) {
   HOLON_CHECK(mfma_serves(head_dim, page_size), "attention (matrix cores): head_dim %d / page %d not served", head_dim,
               page_size);
   HOLON_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && window >= 0 && table_stride > 0,
               "attention: bad sizes");
-  HOLON_CHECK(v_share >= 1 && kv_heads % v_share == 0 && (v_share == 1 || fused == nullptr),
+  HOLON_CHECK(v_share >= 1 && kv_heads % v_share == 0 && ((v_share == 1 && hgate == nullptr) || fused == nullptr),
               "attention: %d key heads do not share value heads by %d", kv_heads, v_share);
+  HOLON_CHECK(hgate == nullptr || hgate_stride >= heads, "attention: gates %lld apart for %d heads",
+              (long long)hgate_stride, heads);
   HOLON_CHECK(splits > 0 && splits <= 64 && keys_per_split > 0 && keys_per_split % 32 == 0,
               "attention decode: %d splits of %d keys (1 to 64 splits of a multiple of 32 keys)", splits, keys_per_split);
   HOLON_CHECK(waves >= 1 && waves <= 8 && splits % waves == 0 && (waves - 1) * (16 * head_dim + 32) * 4 <= 64 * 1024,
@@ -2080,6 +2091,7 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
   a.scale_log2 = scale * 1.4426950408889634f; a.window = window;
   a.part_o = part_o; a.part_ml = part_ml; a.splits = splits; a.keys_per_split = keys_per_split;
   a.out_splits = splits / waves; a.rows_in_order = rows_in_order; a.sink = sink; a.v_share = v_share;
+  a.hgate = (const bf16_t*)hgate; a.hgate_stride = hgate_stride;
   const TileMap tm = tile_map(heads / kv_heads);
   dim3 grid(a.out_splits, kv_heads * tm.head_blocks, n_rows);
   hipStream_t s = (hipStream_t)stream;
@@ -2109,11 +2121,14 @@ static int decode_launch(const void* q, void* out, const void* pages, const int3
   splits = a.out_splits;
   dim3 mgrid(n_rows, heads);
   if (head_dim == 64)
-    attn_merge_kernel<64><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits, sink);
+    attn_merge_kernel<64><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits, sink,
+                                                 a.hgate, a.hgate_stride);
   else if (head_dim == 128)
-    attn_merge_kernel<128><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits, sink);
+    attn_merge_kernel<128><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits, sink,
+                                                 a.hgate, a.hgate_stride);
   else
-    attn_merge_kernel<256><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits, sink);
+    attn_merge_kernel<256><<<mgrid, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, row_ids, query_start, heads, splits, sink,
+                                                 a.hgate, a.hgate_stride);
   HOLON_LAUNCH_OK();
   return 0;
 }
@@ -2184,21 +2199,22 @@ extern "C" int holon_attention_prefill_mod_bf16(const void* q, void* out, const 
                         heads, kv_heads, head_dim, page_size, scale, window, sink, stream, &mod);
 }
 
-// Prompt portions and decode rows over pages whose key heads share value heads: a page holds kv_heads planes of keys,
-// then kv_heads / v_share planes of values, and key head hk reads value head hk / v_share (several score maps over one
-// set of values). With a sink (nullable) and changed scores (softcap 0, r1 and r2 null, keep_first 0: none).
+// Prompt portions and decode rows with every option: v_share > 1: a page holds kv_heads planes of keys, then kv_heads /
+// v_share planes of values, and key head hk reads value head hk / v_share (several score maps over one set of values);
+// a sink (nullable); changed scores (softcap 0, r1 and r2 null, keep_first 0: none); hgate (nullable): one gate a
+// (token, head), rows hgate_stride apart, whose sigmoid multiplies the head's result.
 extern "C" int holon_attention_prefill_shared_bf16(const void* q, void* out, const void* pages, const int32_t* table,
                                                    int table_stride, const int32_t* slots, const int32_t* lens,
                                                    const int32_t* query_start, const int32_t* row_ids, int n_rows,
                                                    int max_query, int max_len, int heads, int kv_heads, int head_dim,
                                                    int page_size, float scale, int window, const float* sink,
                                                    float softcap, const float* r1, const float* r2, int keep_first,
-                                                   int v_share, void* stream) {
+                                                   int v_share, const void* hgate, int64_t hgate_stride, void* stream) {
   const ScoreMod mod{softcap, r1, r2, keep_first};
   const bool changed = softcap > 0.f || r1 != nullptr || (window > 0 && keep_first > 0);
   return prefill_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_query, max_len,
                         heads, kv_heads, head_dim, page_size, scale, window, sink, stream, changed ? &mod : nullptr,
-                        v_share);
+                        v_share, hgate, hgate_stride);
 }
 
 extern "C" int holon_attention_decode_shared_bf16(const void* q, void* out, const void* pages, const int32_t* table,
@@ -2208,12 +2224,12 @@ extern "C" int holon_attention_decode_shared_bf16(const void* q, void* out, cons
                                                   float scale, int window, float* part_o, float* part_ml, int splits,
                                                   int keys_per_split, int waves, int rows_in_order, const float* sink,
                                                   float softcap, const float* r1, const float* r2, int keep_first,
-                                                  int v_share, void* stream) {
+                                                  int v_share, const void* hgate, int64_t hgate_stride, void* stream) {
   const ScoreMod mod{softcap, r1, r2, keep_first};
   const bool changed = softcap > 0.f || r1 != nullptr || (window > 0 && keep_first > 0);
   return decode_launch(q, out, pages, table, table_stride, slots, lens, query_start, row_ids, n_rows, max_len, heads,
                        kv_heads, head_dim, page_size, scale, window, part_o, part_ml, splits, keys_per_split, stream,
-                       nullptr, waves, rows_in_order, sink, changed ? &mod : nullptr, v_share);
+                       nullptr, waves, rows_in_order, sink, changed ? &mod : nullptr, v_share, hgate, hgate_stride);
 }
 
 // Decode rows straight from the step's raw q/k/v projection: per-head norm, rotation and the cache write of each

@@ -83,20 +83,24 @@ int holon_attention_decode_sink_bf16(const void* q, void* out, const void* pages
                                      float* part_o, float* part_ml, int splits, int keys_per_split, int waves,
                                      int rows_in_order, const float* sink, void* stream);
 // Both over pages whose key heads share value heads: kv_heads planes of keys, then kv_heads / v_share planes of values
-// a page; key head hk reads value head hk / v_share. Sink nullable; softcap 0, r1 = r2 = null, keep_first 0: plain scores.
+// a page; key head hk reads value head hk / v_share (1: as ever). Sink nullable; softcap 0, r1 = r2 = null,
+// keep_first 0: plain scores. hgate (nullable, bfloat16, rows hgate_stride apart): head h's result of token t times
+// sigmoid(hgate[t, h]).
 int holon_attention_prefill_shared_bf16(const void* q, void* out, const void* pages, const int32_t* table,
                                         int table_stride, const int32_t* slots, const int32_t* lens,
                                         const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_query,
                                         int max_len, int heads, int kv_heads, int head_dim, int page_size, float scale,
                                         int window, const float* sink, float softcap, const float* r1, const float* r2,
-                                        int keep_first, int v_share, void* stream);
+                                        int keep_first, int v_share, const void* hgate, int64_t hgate_stride,
+                                        void* stream);
 int holon_attention_decode_shared_bf16(const void* q, void* out, const void* pages, const int32_t* table,
                                        int table_stride, const int32_t* slots, const int32_t* lens,
                                        const int32_t* query_start, const int32_t* row_ids, int n_rows, int max_len,
                                        int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
                                        float* part_o, float* part_ml, int splits, int keys_per_split, int waves,
                                        int rows_in_order, const float* sink, float softcap, const float* r1,
-                                       const float* r2, int keep_first, int v_share, void* stream);
+                                       const float* r2, int keep_first, int v_share, const void* hgate,
+                                       int64_t hgate_stride, void* stream);
 // The same from the step's raw q/k/v projection `qkv` [T, (heads + 2 kv_heads) head_dim]: per-head RMSNorm (q_weight
 // and k_weight, both or neither), rotation (rope_table [max_positions, head_dim] = cos | sin, or NULL) and the cache
 // write of every row's new token (write_page, write_off by token; its position is the row's len - 1) happen inside

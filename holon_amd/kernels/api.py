@@ -141,7 +141,8 @@ class Kernels(Protocol):
     def paged_attention(self, q: torch.Tensor, pages: torch.Tensor, table: torch.Tensor, rows: AttnRows,
                         page_size: int, scale: float, window: int, sink: torch.Tensor | None = None,
                         softcap: float = 0.0, dist: tuple[torch.Tensor, torch.Tensor] | None = None,
-                        keep_first: int = 0, value_share: int = 1) -> torch.Tensor:
+                        keep_first: int = 0, value_share: int = 1, head_gate: torch.Tensor | None = None
+                        ) -> torch.Tensor:
         """softmax(q k^T * scale) v per row over its cached tokens, causal; with window W > 0 a query at position p
         sees keys p-W+1 .. p. q [T, Hq, D] -> [T, Hq, D]. This step's keys are already in the cache. `sink` [Hq]
         float32: exp(sink[h] - max) is added to the softmax's denominator (it has no key and no value). Where
@@ -149,7 +150,8 @@ class Kernels(Protocol):
         `dist` = (r1 [Hq], r2 [Hq]) float32: s <- s - r1 ln(1 + r2 (p - j)) for the key at position j; `keep_first`:
         under a window, keys 0 .. keep_first - 1 stay visible. `value_share` s > 1 (there as well): `pages` is
         [n, Hkv + Hkv / s, P * D], Hkv planes of keys and then Hkv / s of values, and key head h reads value head
-        h // s (several score maps over one set of values)."""
+        h // s (several score maps over one set of values). `head_gate` [T, Hq] (there as well; columns of wider rows
+        will do): head h's result of token t is multiplied by sigmoid(head_gate[t, h]) before it is rounded."""
 
     def qkv_attention(self, qkv: torch.Tensor, heads: int, kv_heads: int, head_dim: int,
                       q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float,

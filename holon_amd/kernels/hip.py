@@ -83,9 +83,9 @@ class HipKernels:
             "holon_attention_decode_mod_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
                                                 _P, _P, _I, _I, _I, _I, _P, _F, _P, _P, _I, _P],
             "holon_attention_prefill_shared_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F,
-                                                    _I, _P, _F, _P, _P, _I, _I, _P],
+                                                    _I, _P, _F, _P, _P, _I, _I, _P, _L, _P],
             "holon_attention_decode_shared_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
-                                                   _P, _P, _I, _I, _I, _I, _P, _F, _P, _P, _I, _I, _P],
+                                                   _P, _P, _I, _I, _I, _I, _P, _F, _P, _P, _I, _I, _P, _L, _P],
             "holon_attention_decode_fused_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I,
                                                   _P, _P, _F, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P],
             "holon_gemm_skinny_supported": [_I, _I, _I],
@@ -647,14 +647,14 @@ class HipKernels:
         return bool(dtype in _DT and self.lib.holon_attention_mfma_supported(head_dim, page_size, _DT[dtype]))
 
     def paged_attention(self, q, pages, table, rows: AttnRows, page_size, scale, window, sink=None, softcap=0.0,
-                        dist=None, keep_first=0, value_share=1):
+                        dist=None, keep_first=0, value_share=1, head_gate=None):
         self._check(q, "attention q")
         self._check(pages, "attention pages", q.dtype)
         self._check(table, "block table", torch.int32)
         t, hq, d = q.shape
-        if value_share > 1:
+        if value_share > 1 or head_gate is not None:
             return self._shared_attention(q, pages, table, rows, page_size, scale, window, sink, softcap, dist,
-                                          keep_first, int(value_share))
+                                          keep_first, int(value_share), head_gate)
         hkv = pages.shape[2]
         if pages.shape[1] != 2 or pages.shape[3] != page_size * d:
             raise KernelError(f"attention: pages {tuple(pages.shape)} do not fit head_dim {d}, page {page_size}")
@@ -716,14 +716,21 @@ class HipKernels:
                    self._stream())
         return out
 
-    def _shared_attention(self, q, pages, table, rows, page_size, scale, window, sink, softcap, dist, keep_first, share):
-        """`paged_attention` over pages [n, Hkv + Hkv / share, P * D] whose key heads share value heads: the
-        matrix-core kernels alone (a caller asks `attention_on_cores` first)."""
+    def _shared_attention(self, q, pages, table, rows, page_size, scale, window, sink, softcap, dist, keep_first, share,
+                          head_gate=None):
+        """`paged_attention` over pages [n, Hkv + Hkv / share, P * D] whose key heads share value heads, and with a
+        gate a (token, head): the matrix-core kernels alone (a caller asks `attention_on_cores` first)."""
         t, hq, d = q.shape
+        if share == 1 and pages.dim() == 4 and pages.shape[1] == 2:
+            pages = pages.view(pages.shape[0], 2 * pages.shape[2], pages.shape[3])
         if pages.dim() != 3 or pages.shape[2] != page_size * d or pages.shape[1] % (share + 1):
             raise KernelError(f"attention: pages {tuple(pages.shape)} do not hold key heads that share value heads by "
                               f"{share} at head_dim {d}, page {page_size}")
         hkv = pages.shape[1] // (share + 1) * share
+        if head_gate is not None and not (head_gate.is_cuda and head_gate.dtype == q.dtype and head_gate.shape == (t, hq)
+                                          and head_gate.stride(1) == 1):
+            raise KernelError(f"attention: gates {tuple(head_gate.shape)} {head_gate.dtype} (strides "
+                              f"{head_gate.stride()}) for {t} tokens of {hq} heads")
         if not self.lib.holon_attention_mfma_supported(d, page_size, self._dt(q, "attention")) or hq % hkv:
             raise KernelError(f"attention: shared value heads are served by the matrix-core kernels, not at head_dim "
                               f"{d}, page {page_size}, {q.dtype}, {hq}/{hkv} heads")
@@ -736,7 +743,8 @@ class HipKernels:
         common = (q.data_ptr(), out.data_ptr(), pages.data_ptr(), table.data_ptr(), table.shape[1],
                   rows.slots.data_ptr(), rows.lens.data_ptr(), rows.query_start.data_ptr())
         mod = (float(softcap), _ptr(dist[0]) if dist is not None else None,
-               _ptr(dist[1]) if dist is not None else None, int(keep_first) if window > 0 else 0, share)
+               _ptr(dist[1]) if dist is not None else None, int(keep_first) if window > 0 else 0, share,
+               _ptr(head_gate), head_gate.stride(0) if head_gate is not None else 0)
         if rows.n_chunk:
             self._call(self.lib.holon_attention_prefill_shared_bf16, *common, rows.chunk_rows.data_ptr(), rows.n_chunk,
                        rows.max_chunk_query, rows.max_chunk_len, hq, hkv, d, page_size, float(scale), int(window),

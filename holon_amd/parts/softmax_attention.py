@@ -311,27 +311,32 @@ register_kernel(KernelOp("add_bias", add_bias_plain, "holon_add_bias", [_P, _P, 
 
 
 def attend(k, q, held, view, step, kv_heads, vdim, sink, scale, window, softcap=0.0, dist=None, keep_first=0,
-           value_share=1):
+           value_share=1, head_gate=None):
     """The attention of the mixers: on the matrix cores where keys and values have one width that those kernels
     serve (the pages' layout is then theirs), else the general kernel. q [T, H, D] -> [T, H V]. `value_share` s > 1:
-    a page holds kv_heads / s value heads behind its kv_heads key heads, and key head g reads value head g // s."""
+    a page holds kv_heads / s value heads behind its kv_heads key heads, and key head g reads value head g // s.
+    `head_gate` [T, H] (a view with a row stride will do): head h's result is multiplied by sigmoid(head_gate[t, h]),
+    in the matrix-core kernels' last step, else by a kernel of its own behind the general one."""
     t, heads, dim = q.shape
     keep = keep_first if window > 0 else 0
+    more = {} if head_gate is None else {"head_gate": head_gate}       # (only named where there is one)
     if dim == vdim and k.attention_on_cores(dim, view.page_size, q.dtype):
         if value_share > 1:
             pages = held.pages.view(-1, kv_heads + kv_heads // value_share, view.page_size * dim)
             return k.paged_attention(q, pages, view.table, step.rows, view.page_size, scale, window, sink=sink,
-                                     softcap=softcap, dist=dist, keep_first=keep, value_share=value_share
+                                     softcap=softcap, dist=dist, keep_first=keep, value_share=value_share, **more
                                      ).view(t, heads * vdim)
         pages = held.pages.view(-1, 2, kv_heads, view.page_size * dim)
         return k.paged_attention(q, pages, view.table, step.rows, view.page_size, scale, window, sink=sink,
-                                 softcap=softcap, dist=dist, keep_first=keep).view(t, heads * vdim)
+                                 softcap=softcap, dist=dist, keep_first=keep, **more).view(t, heads * vdim)
     if value_share > 1:
-        return k.softmax_attention(q, held.pages, view.table, step.rows, step.token_row, step.positions, kv_heads, vdim,
-                                   view.page_size, sink, scale, window, softcap=softcap, dist=dist, keep_first=keep,
-                                   value_share=value_share)
-    return k.softmax_attention(q, held.pages, view.table, step.rows, step.token_row, step.positions, kv_heads, vdim,
-                               view.page_size, sink, scale, window, softcap=softcap, dist=dist, keep_first=keep)
+        out = k.softmax_attention(q, held.pages, view.table, step.rows, step.token_row, step.positions, kv_heads, vdim,
+                                  view.page_size, sink, scale, window, softcap=softcap, dist=dist, keep_first=keep,
+                                  value_share=value_share)
+    else:
+        out = k.softmax_attention(q, held.pages, view.table, step.rows, step.token_row, step.positions, kv_heads, vdim,
+                                  view.page_size, sink, scale, window, softcap=softcap, dist=dist, keep_first=keep)
+    return out if head_gate is None else k.head_gate(out, head_gate, heads)
 
 
 def to_half_split(rows_per_head: int, heads: int, rot: int) -> torch.Tensor:
@@ -478,10 +483,10 @@ class SoftmaxAttention(Part):
                                step.positions, held.pages, view.write_page, view.write_off, view.page_size,
                                bias=self.bias, values="keys" if self.values_from_keys else "own")
         sink = self.sink if self.has_sink else self.fixed_sink
+        gates = qkv[:, self.qkv_width: self.qkv_width + self.heads] if self.has_gate else None
         out = attend(k, q, held, view, step, self.kv_heads, self.vdim, sink, self.scale,
-                     self.window, self.softcap, (self.r1, self.r2) if self.distance_bias else None, self.keep_first)
-        if self.has_gate:
-            k.head_gate(out, qkv[:, self.qkv_width: self.qkv_width + self.heads], self.heads)
+                     self.window, self.softcap, (self.r1, self.r2) if self.distance_bias else None, self.keep_first,
+                     head_gate=gates)
         out = self.o(out)
         return k.add_bias(out, self.o_bias) if self.has_o_bias and add_row else out
 

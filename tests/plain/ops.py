@@ -171,7 +171,7 @@ class TorchKernels:
         return self.cores
 
     def paged_attention(self, q, pages, table, rows, page_size, scale, window, sink=None, softcap=0.0, dist=None,
-                        keep_first=0, value_share=1):
+                        keep_first=0, value_share=1, head_gate=None):
         t, hq, d = q.shape
         if value_share > 1:                  # [n, Hkv + Hkv / s, P D]: key head h reads value head h // s
             hkv = pages.shape[1] // (value_share + 1) * value_share
@@ -205,7 +205,10 @@ class TorchKernels:
             if sink is not None:             # a column of its own in the softmax, dropped again: it has no value
                 scores = torch.cat((scores, _up(sink)[:, None, None].expand(hq, e - s, 1)), dim=-1)
             probs = scores.softmax(-1)[..., :n]
-            out[s:e] = torch.einsum("hqk,khd->qhd", probs, v).to(q.dtype)
+            mixed = torch.einsum("hqk,khd->qhd", probs, v)
+            if head_gate is not None:
+                mixed = mixed * torch.sigmoid(_up(head_gate[s:e]))[:, :, None]
+            out[s:e] = mixed.to(q.dtype)
         return out
 
     def argmax(self, logits):

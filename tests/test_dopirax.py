@@ -606,7 +606,7 @@ def test_a_shared_prefix_through_the_engine(folders, device):
 @pytest.mark.parametrize("dim", [64, 128, 256])
 def test_the_cap_and_the_fixed_sink_on_the_matrix_cores(dim):
     """`paged_attention` as the attention mixer calls it (all keys before the query, a cap or none, a sink of 0 for
-    every head), in bfloat16 at every head size the matrix cores serve, prompt portions beside decode rows over
+    every head, a gate a head or none), in bfloat16 at every head size the matrix cores serve, prompt portions beside decode rows over
     scattered pages, short rows among them (where the one in the denominator weighs most), against float64."""
     from holon_amd.kernels import load_hip
     from holon_amd.kernels.api import AttnRows
@@ -634,13 +634,20 @@ def test_the_cap_and_the_fixed_sink_on_the_matrix_cores(dim):
                     max_chunk_len=max(lens[b] for b in chunk))
     sink = torch.zeros(heads, device=dev)
     twin = TorchKernels()
+    gates = (2.0 * torch.randn(qstart[-1], heads + 7, generator=g)).to(dev).bfloat16()[:, 3: 3 + heads]    # columns of wider rows
     for scale, cap in ((2.0 * dim ** -0.5, 3.0), (dim ** -0.5, 30.0), (dim ** -0.5, 0.0), (0.05 * dim ** -0.5, 0.0)):
-        got = k.paged_attention(q, pages, table.to(dev), rows, page, scale, 0, sink=sink, softcap=cap)
-        want = twin.paged_attention(q.double(), pages.double(), table.to(dev), rows, page, scale, 0, sink=sink.double(),
-                                    softcap=cap)
-        assert H.rel_rms(got, want) < 8e-3, (dim, scale, cap)
-        per = ((got.double() - want).square().mean((1, 2)).sqrt() / want.square().mean().sqrt()).max().item()
-        assert per < 4e-2, (dim, scale, cap, per)
+        for gate in (None, gates):                 # the gate a head in the kernels' last step
+            got = k.paged_attention(q, pages, table.to(dev), rows, page, scale, 0, sink=sink, softcap=cap, head_gate=gate)
+            want = twin.paged_attention(q.double(), pages.double(), table.to(dev), rows, page, scale, 0,
+                                        sink=sink.double(), softcap=cap, head_gate=None if gate is None else gate.double())
+            assert H.rel_rms(got, want) < 8e-3, (dim, scale, cap)
+            per = ((got.double() - want).square().mean((1, 2)).sqrt() / want.square().mean().sqrt()).max().item()
+            assert per < 4e-2, (dim, scale, cap, per)
+        if cap == 0.0:                             # and without a sink: the kernels that stage keys through LDS
+            got = k.paged_attention(q, pages, table.to(dev), rows, page, scale, 0, head_gate=gates)
+            want = twin.paged_attention(q.double(), pages.double(), table.to(dev), rows, page, scale, 0,
+                                        head_gate=gates.double())
+            assert H.rel_rms(got, want) < 8e-3, (dim, scale, "gate alone")
 
 
 @pytest.mark.gpu
