@@ -1,11 +1,11 @@
 """Dopirax: its typed configuration, and configuration to spec.
 
 A decoder whose two sublayers read one norm of the residual stream, x += mixer(a) + ffn(a) with a = norm(x), the
-stream kept in float32 and the norm an RMS norm whose stored weight lies around zero (it multiplies by 1 + w). The
+stream kept in float32 and the norm an RMS norm whose weight is kept as an offset w from one (it multiplies by 1 + w). The
 embedding's rows are multiplied by a constant. Each layer names its mixer: `attention` (grouped-query softmax
 attention with biases on the query, key and output projections, no value projection (a token's values are its keys
 before the rotation), rotary positions on the first dimensions of a head in the half-split pairing, scores squashed by
-a tanh cap, a softmax with one added to its denominator, and one sigmoid gate a head on the result) or `attention_2`
+a tanh cap, a softmax whose denominator holds one more term, exp(0), and one sigmoid gate a head on the result) or `attention_2`
 (differential attention: two softmax maps a head over one set of values, queries and keys RMS-normed per head and map
 and turned in the interleaved pairing, the second map's result taken off the first's with a factor the layer learns,
 the difference divided by its root mean square; such a layer may have no keys and values of its own and read those an

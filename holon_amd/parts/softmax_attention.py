@@ -360,7 +360,7 @@ class SoftmaxAttention(Part):
     key j for query i (`r1`, `r2`, one number a head each); `keep_first`: under a window the first tokens of the
     sequence stay visible, at their true positions.
 
-    `values_from_keys`: there is no value projection; a token's values are its keys as projected (bias added, before
+    `values_from_keys`: there is no value projection; a token's values are its keys straight from the projection (bias added, before
     the rotation), so vdim = dim, and the cache holds the turned key and the unturned one side by side. `sink_value`
     (a number): a sink that every head shares and no tensor holds (0: one is added to the softmax's denominator).
     `head_gate`: a projection `g` of one number a head, computed with q and k in the merged product; head h's result

@@ -131,7 +131,7 @@ def draw(name: str, shape: tuple[int, ...], g: torch.Generator, sharp: bool) -> 
     elif name.endswith("k.norm"):
         x = 1 + 0.15 * n()
     elif last in ("norm1", "norm"):
-        x = 0.3 * n()                                         # stored around zero: the norm multiplies by 1 + w
+        x = 0.3 * n()                                         # an offset from one: the norm multiplies by 1 + w
     elif last == "b" and ".mix." in name:
         x = 0.3 * n()
     elif last == "b":                                         # the router's bias

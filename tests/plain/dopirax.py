@@ -5,7 +5,7 @@ Notation: x [n, W] the residual stream of a sequence of n tokens at positions 0 
 names to tensors; `p` is a tensor name prefix; a = N(x) (1 + g) with N(v) = v / sqrt(mean(v^2) + eps).
 
   layer           x <- x + (mixer(a) + ffn(a)): one norm, read by both sublayers
-  attention       q = Wq a + bq, k = Wk a + bk, v = k (as projected, not turned); q, k turned on their first `dims`
+  attention       q = Wq a + bq, k = Wk a + bk, v = k (from the projection, not turned); q, k turned on their first `dims`
                   dimensions in the pairing (i, i + dims / 2); s_ij = cap tanh(scale q_i . k_j / cap), j <= i;
                   p_ij = exp(s_ij) / (1 + sum_j exp(s_ij)); head h's result times sigmoid(Wg a)_h; Wo (.) + bo
   attention_2     two maps a head: q [H, 2, dim], k [G, 2, dim], v [G, vdim]; per (head, map) q <- N(q) gq, k <- N(k) gk,

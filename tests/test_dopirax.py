@@ -256,7 +256,7 @@ def test_a_far_key_at_a_page_border(tmp_path, kind, dim, page, key_at, dtype, de
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_the_one_in_the_denominator(folders, tmp_path, dtype, device):
-    """The softmax with one added to its denominator: on the first tokens of a sequence (where it weighs most) and
+    """The softmax whose denominator holds one more term, exp(0): on the first tokens of a sequence (where it weighs most) and
     behind scores pushed far below zero (where it takes nearly everything), the plain model with and without it are far
     apart and the engine follows the one with it."""
     cfg, seed, sharp, page = MODELS["attention"]
